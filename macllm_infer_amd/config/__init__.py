@@ -1,19 +1,22 @@
-from .spec import (AttentionSpec, ClampedGLUSpec, ConfigError, GeneralDeltaSpec, HashedBigramSpec, InterleavedRopeSpec,
+from .spec import (AttentionSpec, ClampedGLUSpec, ConfigError, GatedLinearAttentionSpec, GeneralDeltaSpec, HashedBigramSpec,
+                   InterleavedRopeSpec,
                    LatentAttentionSpec, LayerNormSpec, LayerSpec, LogDistanceBiasSpec, Mamba2Spec, MixerSlot,
                    ModelSpec, NoPositionSpec, PolyNormFFNSpec, RetentionSpec, RmsNormSpec, RopeSpec,
-                   RoutedExpertsSpec, ScheduleEntry, StreamInjection, SwiGLUSpec)
+                   RoutedExpertsSpec, ScheduleEntry, StreamInjection, SwiGLUSpec, WavelengthScalingSpec)
 from .registry import (config_from_dict, load_config, register_architecture,
                        registered_architectures)
 from .falcon_h1 import FalconH1Config
 from .mukutar import MukutarConfig
 from .lutosun import LutosunConfig
+from .motolix import MotolixConfig
 
 register_architecture(FalconH1Config)
 register_architecture(MukutarConfig)
 register_architecture(LutosunConfig)
+register_architecture(MotolixConfig)
 
-__all__ = ["AttentionSpec", "ClampedGLUSpec", "ConfigError", "FalconH1Config", "GeneralDeltaSpec", "HashedBigramSpec",
+__all__ = ["AttentionSpec", "ClampedGLUSpec", "ConfigError", "FalconH1Config", "GatedLinearAttentionSpec", "GeneralDeltaSpec", "HashedBigramSpec",
            "InterleavedRopeSpec", "LatentAttentionSpec", "LayerNormSpec", "LayerSpec", "LogDistanceBiasSpec", "LutosunConfig",
-           "Mamba2Spec", "MixerSlot", "ModelSpec", "MukutarConfig", "NoPositionSpec", "PolyNormFFNSpec", "RetentionSpec",
-           "RmsNormSpec", "RopeSpec", "RoutedExpertsSpec", "ScheduleEntry", "StreamInjection", "SwiGLUSpec",
+           "Mamba2Spec", "MixerSlot", "ModelSpec", "MotolixConfig", "MukutarConfig", "NoPositionSpec", "PolyNormFFNSpec", "RetentionSpec",
+           "RmsNormSpec", "RopeSpec", "RoutedExpertsSpec", "ScheduleEntry", "StreamInjection", "SwiGLUSpec", "WavelengthScalingSpec",
            "config_from_dict", "load_config", "register_architecture", "registered_architectures"]

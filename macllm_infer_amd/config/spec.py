@@ -27,11 +27,27 @@ def _require(condition: bool, message: str) -> None:
 
 
 @dataclass(frozen=True)
+class WavelengthScalingSpec:
+    """Frequencies stretched by their wavelength l = 2 pi / f against a context of ``original`` tokens: kept where
+    l < original / high, divided by ``factor`` where l > original / low, and between the two blended,
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    factor: float
+    low: float
+    high: float
+    original: float
+
+    def validate(self) -> None:
+        _require(self.factor > 0 and self.original > 0, "rope scaling needs a positive factor and original context")
+        _require(self.high != self.low, "rope scaling needs two different bounds (low, high)")
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Half-split rotary position encoding of the first ``rotary_dim`` dims of a head
-    (src/architecture.rs:44-62)."""
+    (src/architecture.rs:44-62).  ``scaling``: the frequencies are stretched by wavelength (None: as they are)."""
     theta: float
     rotary_dim: int
+    scaling: Optional[WavelengthScalingSpec] = None
     kind: str = "rope"
 
     def validate(self, head_dim: int) -> None:
@@ -39,6 +55,8 @@ class RopeSpec:
                  f"rope theta must be finite and positive, got {self.theta}")
         _require(0 < self.rotary_dim <= head_dim and self.rotary_dim % 2 == 0,
                  f"rotary_dim {self.rotary_dim} must be even and in 2..={head_dim}")
+        if self.scaling is not None:
+            self.scaling.validate()
 
 
 @dataclass(frozen=True)
@@ -122,6 +140,21 @@ class AttentionSpec:
     out_multiplier: float = 1.0
     value_dim: Optional[int] = None      # width of a value head (None: the keys' head_dim)
     sink: bool = False                   # one more term exp(sink[head]) in the softmax's denominator (tensor ``sink``)
+    # the values are the keys as projected (before any norm's successor, rotation or scaling of the keys): no v_proj
+    values_from_keys: bool = False
+    # a learned number per query head that multiplies its scores (tensor ``temp``)
+    head_temperature: bool = False
+    # "softmax": weights normalized over the visible keys; "sigmoid": every visible key weighs
+    # sigmoid(score + score_bias[head]) on its own, nothing is normalized (tensor ``pb`` when ``score_bias``)
+    weighting: str = "softmax"
+    score_bias: bool = False
+    # RMS norm (plain weights ``q_norm`` / ``k_norm``, this eps) over ALL rows of the q projection at once, and of
+    # the k projection, before the heads are split and before rotation; None: no such norm
+    projection_norm_eps: Optional[float] = None
+    # values are turned by their position over all their dims (half-split pairs, angle = position *
+    # value_rotation_theta^(-2m / value width)) before they are cached, and every head's output is turned back by
+    # its query's position; None: values as projected
+    value_rotation_theta: Optional[float] = None
     kind: str = "attention"
 
     @property
@@ -139,6 +172,15 @@ class AttentionSpec:
                  f"head_dim {self.head_dim} must be positive and even")
         _require(self.scale > 0, "attention scale must be positive")
         _require(self.window is None or self.window > 0, "attention window must be positive")
+        _require(self.weighting in ("softmax", "sigmoid"), f"attention weighting {self.weighting!r} is not known")
+        _require(not self.score_bias or self.weighting == "sigmoid", "a bias per head is for sigmoid weights")
+        _require(not (self.sink and self.weighting == "sigmoid"), "a sink belongs to a softmax")
+        _require(not self.values_from_keys or self.value_width == self.head_dim,
+                 "values that are the keys have the keys' width")
+        _require(self.projection_norm_eps is None or self.projection_norm_eps > 0, "the projections' norm eps must be positive")
+        if self.value_rotation_theta is not None:
+            _require(self.value_rotation_theta > 0 and self.value_width % 2 == 0,
+                     "turned values need a positive base and an even width")
         self.position.validate(self.head_dim)
 
 
@@ -235,11 +277,14 @@ class HashedBigramSpec:
 
 @dataclass(frozen=True)
 class StreamInjection:
-    """What is added to the residual stream right before a schedule entry runs: the embedding output once more
-    (``embedding``), and row ``row`` of the tensor ``vector_name`` [rows, hidden] (None: no vector)."""
+    """What happens to the residual stream right before a schedule entry runs: with ``mix_name`` the stream x
+    becomes W [x; x0], W the tensor ``mix_name`` [hidden, 2 hidden] and x0 the embedding output; then the embedding
+    output is added once more (``embedding``), and row ``row`` of the tensor ``vector_name`` [rows, hidden]
+    (None: no vector)."""
     embedding: bool = False
     vector_name: Optional[str] = None
     row: int = 0
+    mix_name: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -330,6 +375,31 @@ class GeneralDeltaSpec:
 
 
 @dataclass(frozen=True)
+class GatedLinearAttentionSpec:
+    """Linear attention whose state decays per key channel by a gate of the token: per head
+    S <- diag(alpha) S + k v^T, o = S^T q, with q = (W_q h) * ``query_scale``, k = W_k h, v = W_v h and
+    alpha = sigmoid(z)^(1 / ``decay_temperature``), z = W_a2 (W_a1 h) + bias, one number per head and key channel.
+    Each head's o is divided by its root mean square (``norm_eps``) and multiplied by a weight of ``value_dim``
+    numbers that all heads share, then by SiLU of a gate projection, and projected out.  ``decay_rank``: the inner
+    width of the gate's two projections (None: whatever the stored tensors have)."""
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay_temperature: float
+    query_scale: float
+    norm_eps: float
+    decay_rank: Optional[int] = None
+    kind: str = "gated_linear_attention"
+
+    def validate(self) -> None:
+        _require(self.num_heads > 0 and self.key_dim > 0 and self.value_dim > 0,
+                 "gated linear attention sizes must be positive")
+        _require(self.decay_temperature > 0, "the decay's temperature must be positive")
+        _require(self.decay_rank is None or self.decay_rank > 0, "the decay's inner width must be positive")
+        _require(self.norm_eps > 0, "the norm eps must be positive")
+
+
+@dataclass(frozen=True)
 class PolyNormFFNSpec:
     """down(act(up(x))) with act(z) = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers element by element, N the
     division of a token's row by its root mean square (``eps``); the four numbers are the tensor ``act``."""
@@ -344,22 +414,27 @@ class PolyNormFFNSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """down(SiLU(gate(x) * gate_multiplier) * up(x)) * down_multiplier (src/decoder.rs:261-306)."""
+    """down(act(gate(x) * gate_multiplier) * up(x)) * down_multiplier (src/decoder.rs:261-306), act = SiLU or,
+    with ``activation`` "gelu_tanh", 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
     intermediate_size: int
     bias: bool = False
     gate_multiplier: float = 1.0
     down_multiplier: float = 1.0
+    activation: str = "silu"
     kind: str = "swiglu"
 
     def validate(self) -> None:
         _require(self.intermediate_size > 0, "intermediate_size must be positive")
+        _require(self.activation in ("silu", "gelu_tanh"), f"the gate's activation {self.activation!r} is not known")
 
 
 @dataclass(frozen=True)
 class MixerSlot:
-    """One mixer of a layer: the sub-path of its tensors and its spec."""
+    """One mixer of a layer: the sub-path of its tensors and its spec.  ``weight``: the number its output is
+    multiplied by (in float32) where the layer's mixers are summed."""
     name: str
     spec: object
+    weight: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -388,6 +463,12 @@ class LayerSpec:
     ffn_scale_name: Optional[str] = None
     # one number that multiplies every branch where it joins the stream (x <- x + m * branch), applied in float32
     branch_multiplier: float = 1.0
+    # arrangement "sandwich": a second norm on each branch before it joins the stream,
+    # x <- x + mixer_post_norm(sum of mixers(mixer_norm(x))), x <- x + ffn_post_norm(ffn(ffn_norm(x)))
+    mixer_post_norm: object = None
+    ffn_post_norm: object = None
+    mixer_post_norm_name: str = "norm1b"
+    ffn_post_norm_name: str = "norm2b"
 
 
 @dataclass(frozen=True)
@@ -419,6 +500,8 @@ class ModelSpec:
     bigram_name: str = "bigram"
     # tensors [rows, hidden] that schedule entries name (``StreamInjection.vector_name``): (name, rows)
     injected_vectors: Tuple[Tuple[str, int], ...] = ()
+    # tensors [hidden, 2 hidden] that schedule entries name (``StreamInjection.mix_name``)
+    injected_mixes: Tuple[str, ...] = ()
     embedding_name: str = "model.embed_tokens"
     final_norm_name: str = "model.norm"
     lm_head_name: str = "lm_head"
@@ -459,6 +542,9 @@ class ModelSpec:
                 _require(entry.before.vector_name in vectors
                          and 0 <= entry.before.row < vectors[entry.before.vector_name],
                          f"schedule entry {index} adds a row of a vector table that the model does not have")
+            if entry.before is not None and entry.before.mix_name is not None:
+                _require(entry.before.mix_name in self.injected_mixes,
+                         f"schedule entry {index} mixes the stream with a matrix that the model does not have")
         for layer in self.layers:
             _require(len(layer.mixers) > 0, f"layer {layer.prefix} has no mixer")
             names = [slot.name for slot in layer.mixers]
@@ -466,9 +552,13 @@ class ModelSpec:
             for slot in layer.mixers:
                 slot.spec.validate()
             layer.mixer_norm.validate()
+            if layer.mixer_post_norm is not None:
+                layer.mixer_post_norm.validate()
             if layer.ffn is not None:
                 layer.ffn.validate()
                 layer.ffn_norm.validate()
+                if layer.ffn_post_norm is not None:
+                    layer.ffn_post_norm.validate()
         for index, entry in enumerate(self.schedule):
             _require(0 <= entry.layer < len(self.layers),
                      f"schedule entry {index} names layer {entry.layer}, which does not exist")

@@ -13,6 +13,8 @@ from ..kernels import ops
 from ..cache.manager import StateNeed
 from ..parts.base import BuildContext, Residual, RowVector, WeightedBranch, part_class
 from ..parts.block import arrangement_class
+from ..parts.linear import Linear
+from ..parts.norm import fold_pending
 from ..weights.loader import Expect
 
 
@@ -37,6 +39,8 @@ class DecoderModel:
             out.append(Expect(f"{spec.bigram_name}.weight", ((spec.bigram.buckets + 1, spec.hidden_size),), init="embedding"))
         for name, rows in spec.injected_vectors:
             out.append(Expect(name, ((rows, spec.hidden_size),), init="bias"))
+        for name in spec.injected_mixes:
+            out.append(Expect(name, ((spec.hidden_size, 2 * spec.hidden_size),)))
         for layer in spec.layers:
             out += arrangement_class(layer.arrangement).expected_tensors(layer, spec.hidden_size)
         out += part_class(spec.final_norm).expected_tensors(spec.final_norm, spec.final_norm_name, spec.hidden_size)
@@ -102,6 +106,8 @@ class DecoderModel:
         self.injected = {name: tensors[name].to(torch.float32).contiguous().to(build.device)
                          for name, _ in spec.injected_vectors}
         self._keeps_embedding = any(entry.before is not None and entry.before.embedding for entry in spec.schedule)
+        # the matrices W of the entries that turn the stream x into W [x; x0]
+        self.mixes = {name: Linear([tensors[name]], [None], build) for name in spec.injected_mixes}
         self.blocks = [arrangement_class(layer.arrangement)(layer, tensors, build) for layer in spec.layers]
         for block in self.blocks:                    # what a layer decides by timing itself among the others
             tune = getattr(block, "tune", None)
@@ -164,12 +170,23 @@ class DecoderModel:
                              spec.bigram.mul_prev, spec.bigram.mul_cur, step.positions, step.lane_of_token,
                              step.cu_seqlens, step.slot_ids, cache.entry(MODEL_STATE).states["previous_token"], h)
         embedded = h.clone() if self._keeps_embedding else None
+        beside = None
+        if self.mixes:
+            # [x | x0] in the activation dtype: the embedding output is laid into the right half once
+            width = spec.hidden_size
+            beside = torch.empty((step.num_tokens, 2 * width), dtype=self.build.dtype, device=self.build.device)
+            ops.cast_rows(h, beside[:, width:])
         residual = Residual(h)
         for index, entry in enumerate(spec.schedule):
             block = self.blocks[entry.layer]
             if entry.before is not None:
                 # what joins the stream before this run waits with the branches of the run before it: the run's
                 # first norm adds them all in its own launch
+                if entry.before.mix_name is not None:
+                    # x <- W [x; x0]: the stream as it is behind everything pending, the sums kept in float32
+                    fold_pending(residual)
+                    ops.cast_rows(residual.h, beside[:, :spec.hidden_size])
+                    residual.h = ops.linear(beside, self.mixes[entry.before.mix_name].weight, None, keep_float32=True)
                 added = list(residual.pending)
                 if entry.before.embedding:
                     added.append(WeightedBranch(embedded, 1.0))

@@ -36,7 +36,8 @@ _SIGNATURES = {
                            _c_int, _c_ptr],
         "mi_add_partials_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
                                     _c_int, _c_ptr],
-        "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+        "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+        "mi_cast_rows": [_c_ptr, _c_ptr, _c_int, _c_long, _c_int, _c_int, _c_ptr],
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
         "mi_tanh_softcap": [_c_ptr, _c_float, _c_long, _c_ptr],
         "mi_add_bias_round": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -47,7 +48,8 @@ _SIGNATURES = {
                             _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_stream_add": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_add_layernorm": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr,
-                             _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+                             _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
+                             _c_ptr],
         "mi_clamped_glu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr],
     },
     "latent": {
@@ -76,11 +78,11 @@ _SIGNATURES = {
     "linear_state": {
         "mi_linear_state_scan": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
                                  _c_ptr, _c_ptr, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int,
-                                 _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_ptr],
+                                 _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_float, _c_float, _c_ptr],
         "mi_linear_state_scan_chunked": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                          _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_float, _c_ptr,
-                                         _c_ptr, _c_int, _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr,
-                                         _c_int, _c_ptr, _c_ptr, _c_ptr],
+                                         _c_ptr, _c_int, _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_float, _c_float,
+                                         _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
         "mi_linear_state_local_floats": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "mi_linear_state_start_floats": [_c_int, _c_int, _c_int, _c_int],
         "mi_head_norm_gate": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr,
@@ -92,7 +94,11 @@ _SIGNATURES = {
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
                                _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                               _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+                               _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                               _c_ptr],
+        "mi_attention_prepare": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                                 _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int,
+                                 _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
@@ -303,16 +309,33 @@ def add_partials_rmsnorm(h: torch.Tensor, partial: torch.Tensor, weight: torch.T
         None, T, T, d, _stream()), "add_partials_rmsnorm", f"(d={d}, S={partial.shape[0]})")
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, tile: int = 0) -> None:
-    """out[t, i] = SiLU(g[t, i]) * u[t, i] with a row of ``gate_up`` holding [g | u] (``tile`` 0) or
-    g and u interleaved in tiles of ``tile`` columns: [g[0:tile] | u[0:tile] | g[tile:2 tile] | ...]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, tile: int = 0, activation: str = "silu") -> None:
+    """out[t, i] = act(g[t, i]) * u[t, i] with a row of ``gate_up`` holding [g | u] (``tile`` 0) or
+    g and u interleaved in tiles of ``tile`` columns: [g[0:tile] | u[0:tile] | g[tile:2 tile] | ...]; act is SiLU
+    or ("gelu_tanh") 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
+    _need(activation in GATE_ACTIVATIONS, f"swiglu: the activation {activation!r} is not known")
     ld = _row_major(gate_up, "gate_up")
     T, two_i = gate_up.shape
     _need(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.is_contiguous() and out.dtype == gate_up.dtype,
           "swiglu: out must be contiguous [T, I] of the input's dtype")
     _need(tile >= 0 and (tile == 0 or (two_i // 2) % tile == 0), "swiglu: the tile must divide the width")
-    _check(_fn("common", "mi_swiglu")(_p(gate_up), _dt(gate_up), ld, _p(out), T, two_i // 2, int(tile), _stream()),
-           "swiglu")
+    _check(_fn("common", "mi_swiglu")(_p(gate_up), _dt(gate_up), ld, _p(out), T, two_i // 2, int(tile),
+                                      GATE_ACTIVATIONS[activation], _stream()), "swiglu")
+
+
+def cast_rows(source: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, :] = source[t, :] in ``out``'s dtype: the float32 stream's rows into (a column block of) a matrix of
+    activations."""
+    _need(source.dtype == torch.float32 and source.dim() == 2 and source.is_contiguous() and source.is_cuda,
+          "cast_rows: the source must be contiguous float32 [T, d] on the GPU")
+    ld = _row_major(out, "out")
+    _need(out.shape == source.shape, "cast_rows: out must have the source's shape")
+    if source.numel():
+        _check(_fn("common", "mi_cast_rows")(_p(source), _p(out), _dt(out), ld, source.shape[0], source.shape[1],
+                                             _stream()), "cast_rows")
 
 
 def scale_to_f32(values: torch.Tensor, multiplier: float, out: torch.Tensor) -> None:
@@ -403,20 +426,28 @@ def stream_add(h: torch.Tensor, rows: Optional[torch.Tensor], factor: float, vec
                                           _p(vector), T, d, _stream()), "stream_add")
 
 
-def add_layernorm(h: torch.Tensor, branches: Sequence[tuple], vector: Optional[torch.Tensor], weight: torch.Tensor,
-                  bias: torch.Tensor, eps: float, out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+def add_layernorm(h: torch.Tensor, branches: Sequence[tuple], vector: Optional[torch.Tensor],
+                  weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                  rows: Optional[torch.Tensor] = None, branch_norm: Optional[tuple] = None) -> None:
     """h += sum of factor * branch over ``branches`` [(tensor [T, d], factor)] (at most three) + ``vector`` [d]
     (float32, in place); out = (h - mean) / sqrt(variance + eps) * weight + bias, statistics in float32, the
     variance from the deviations.  With ``rows`` only those rows are read, ``out[i]`` gets row ``rows[i]`` and
-    ``h`` is left as it is."""
+    ``h`` is left as it is.  ``branch_norm`` (weight, bias, eps): the branches' weighted sum goes through a layer
+    norm of its own before it is added, h += LN(sum) * weight + bias.  Without ``out`` nothing is normed behind
+    the add, and ``weight`` and ``bias`` may be None."""
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and h.is_cuda,
           "add_layernorm: h must be contiguous float32 [T, d]")
     T, d = h.shape
     _need(len(branches) <= 3, "add_layernorm: at most three branches")
     for tensor, _ in branches:
         _need(tensor.shape == h.shape and tensor.is_contiguous(), "add_layernorm: branches must be contiguous [T, d]")
-    for name, one in (("weight", weight), ("bias", bias)):
-        _need(one.dtype == torch.float32 and one.numel() == d and one.is_contiguous(), f"add_layernorm: {name} must be float32 [d]")
+    named = [("weight", weight), ("bias", bias)] if out is not None or weight is not None else []
+    if branch_norm is not None:
+        _need(rows is None and len(branches) > 0, "add_layernorm: a norm on the branches needs branches and all rows")
+        named += [("the branches' weight", branch_norm[0]), ("the branches' bias", branch_norm[1])]
+    for name, one in named:
+        _need(one is not None and one.dtype == torch.float32 and one.numel() == d and one.is_contiguous(),
+              f"add_layernorm: {name} must be float32 [d]")
     _need(vector is None or (vector.dtype == torch.float32 and vector.numel() == d and vector.is_contiguous()),
           "add_layernorm: the vector must be float32 [d]")
     n_rows = T
@@ -435,9 +466,10 @@ def add_layernorm(h: torch.Tensor, branches: Sequence[tuple], vector: Optional[t
             flat += [_p(tensor), _dt(tensor), float(factor)]
         else:
             flat += [None, DT_F32, 0.0]
+    post = branch_norm if branch_norm is not None else (None, None, 0.0)
     _check(_fn("common", "mi_add_layernorm")(
-        _p(h), *flat, _p(vector), _p(weight), _p(bias), float(eps), _p(out), _dt(out) if out is not None else DT_F32,
-        _p(rows), n_rows, d, _stream()), "add_layernorm", f"(d={d})")
+        _p(h), *flat, _p(vector), _p(weight), _p(bias), float(eps), _p(post[0]), _p(post[1]), float(post[2]), _p(out),
+        _dt(out) if out is not None else DT_F32, _p(rows), n_rows, d, _stream()), "add_layernorm", f"(d={d})")
 
 
 def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, up_offset: float, out: torch.Tensor) -> None:
@@ -746,7 +778,8 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
                       key_scale: float = 1.0, positions: Optional[torch.Tensor] = None,
                       inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0, removal_col: int = -1,
                       decay_logits: Optional[torch.Tensor] = None, decay_bias: Optional[torch.Tensor] = None,
-                      decay_floor: float = 0.0, key_eps: float = 0.0, chunks=None) -> None:
+                      decay_floor: float = 0.0, key_eps: float = 0.0, chunks=None, gate_power: float = 0.0,
+                      query_scale: float = 1.0) -> None:
     """The scan of a mixer whose state is a matrix per head, from and into ``state`` [slots, H, dv, dk] (float32, the
     state of a head transposed), for every lane of the step from its slot; ``out`` float32 [T, H * dv] = S^T q.
 
@@ -755,7 +788,9 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
     turned by ``positions`` (``inv_freq``, ``rotary_dim``; None: no rotation) and k multiplied by ``key_scale``.
     Delta rule (``removal_col`` >= 0: the columns of the removal rate's logits; ``decay_logits`` float32 [T, H * dk],
     ``decay_bias`` float32 [H * dk]): w = exp(-decay_floor * sigmoid(logits + bias)), a = sigmoid(removal),
-    u = k / sqrt(sum k^2 + key_eps), S <- diag(w) S - (a u)(u^T S) + k v^T.  ``max_query_len``: the longest lane
+    u = k / sqrt(sum k^2 + key_eps), S <- diag(w) S - (a u)(u^T S) + k v^T.  Gated decay (``gate_power`` > 0, no
+    removal; ``decay_logits`` and ``decay_bias`` as above): w = sigmoid(logits + bias)^gate_power per head and key
+    channel, S <- diag(w) S + k v^T.  ``query_scale`` multiplies q.  ``max_query_len``: the longest lane
     (1 picks small workgroups; 0: not known).  ``chunks`` (a table of the step's lanes cut into chunks: ``chunks``
     int32 [n, 4], ``lane_chunks`` int32 [lanes, 2], ``num_chunks``, ``chunk_size``): the scan runs chunk by chunk in
     three passes (the chunks' own states and transitions side by side, the carry from chunk to chunk, the outputs
@@ -764,6 +799,7 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
     T = u.shape[0]
     H, dk, dv = int(num_heads), int(key_dim), int(value_dim)
     delta = removal_col >= 0
+    gated = not delta and gate_power > 0
     widest = max(q_col + H * dk, k_col + H * dk, v_col + H * dv, removal_col + H * dk if delta else 0)
     _need(min(q_col, k_col, v_col) >= 0 and u.shape[1] >= widest, "linear_state_scan: u is too narrow for its columns")
     _need(state.dtype == torch.float32 and state.dim() == 4 and state.shape[1:] == (H, dv, dk) and state.is_contiguous()
@@ -775,13 +811,13 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
     _need(out.dtype == torch.float32 and out.shape == (T, H * dv) and out.is_contiguous(),
           "linear_state_scan: out must be contiguous float32 [T, H * dv]")
     logits_ld = 0
-    if delta:
+    if delta or gated:
         _need(decay_logits is not None and decay_logits.dtype == torch.float32 and decay_logits.shape == (T, H * dk),
               "linear_state_scan: decay_logits must be float32 [T, H * dk]")
         logits_ld = _row_major(decay_logits, "decay_logits")
         _need(decay_bias is not None and decay_bias.dtype == torch.float32 and decay_bias.numel() == H * dk
               and decay_bias.is_contiguous() and decay_bias.is_cuda, "linear_state_scan: decay_bias must be float32 [H * dk]")
-    else:
+    if not delta and not gated:
         _need(head_decay is not None and head_decay.dtype == torch.float32 and head_decay.numel() == H
               and head_decay.is_cuda, "linear_state_scan: head_decay must be float32 [H] on the GPU")
     if inv_freq is not None:
@@ -794,7 +830,7 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
         count = int(chunks.num_chunks)
         _need(chunks.chunks.numel() >= 4 * count and chunks.lane_chunks.numel() >= 2 * lanes and count > 0,
               "linear_state_scan: the chunk table does not cover the step")
-        floats = _fn("linear_state", "mi_linear_state_local_floats", _c_long)(count, H, dk, dv, int(delta))
+        floats = _fn("linear_state", "mi_linear_state_local_floats", _c_long)(count, H, dk, dv, 1 if delta else 2 if gated else 0)
         local = torch.empty((floats,), dtype=torch.float32, device=u.device)
         start = torch.empty((_fn("linear_state", "mi_linear_state_start_floats", _c_long)(count, H, dk, dv),),
                             dtype=torch.float32, device=u.device)
@@ -803,14 +839,16 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
             _p(cu_seqlens), _p(slot_ids), lanes, _p(out), out.stride(0), int(chunks.chunk_size), _p(head_decay),
             float(key_scale), _p(positions) if inv_freq is not None else None, _p(inv_freq),
             int(rotary_dim) if inv_freq is not None else 0, _p(decay_logits), logits_ld, _p(decay_bias),
-            float(decay_floor), float(key_eps), _p(chunks.chunks), _p(chunks.lane_chunks), count, _p(local), _p(start),
+            float(decay_floor), float(key_eps), float(gate_power) if gated else 0.0, float(query_scale),
+            _p(chunks.chunks), _p(chunks.lane_chunks), count, _p(local), _p(start),
             _stream()), "linear_state_scan_chunked", f"(dk={dk}, dv={dv}, chunks={count})")
         return
     _check(_fn("linear_state", "mi_linear_state_scan")(
         _p(u), _dt(u), ld, int(q_col), int(k_col), int(v_col), int(removal_col), H, dk, dv, _p(state), _p(cu_seqlens),
         _p(slot_ids), lanes, _p(out), out.stride(0), int(max_query_len), _p(head_decay), float(key_scale),
         _p(positions) if inv_freq is not None else None, _p(inv_freq), int(rotary_dim) if inv_freq is not None else 0,
-        _p(decay_logits), logits_ld, _p(decay_bias), float(decay_floor), float(key_eps), _stream()),
+        _p(decay_logits), logits_ld, _p(decay_bias), float(decay_floor), float(key_eps),
+        float(gate_power) if gated else 0.0, float(query_scale), _stream()),
         "linear_state_scan", f"(dk={dk}, dv={dv})")
 
 
@@ -921,7 +959,8 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                     slopes: Optional[torch.Tensor] = None, query_tiles: Optional[torch.Tensor] = None,
                     tile_tokens: int = 0, cu_seqlens: Optional[torch.Tensor] = None,
                     log_bias: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
-                    value_dim: Optional[int] = None) -> None:
+                    value_dim: Optional[int] = None, head_scales: Optional[torch.Tensor] = None,
+                    score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
@@ -934,7 +973,9 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     tokens, a kernel that fetches a run of keys once for sixteen queries (the same bits as without).
     ``log_bias`` (float32 [Hq, 2] = (r1, r2)): ``score -= r1 * ln(1 + r2 * (s - p))``.  ``sinks`` (float32 [Hq]):
     exp(sink) is one more term of the softmax's denominator, with no key and no value.  ``value_dim``: the
-    width of a value head if it is not the keys'; ``out`` is then [T, Hq * value_dim]."""
+    width of a value head if it is not the keys'; ``out`` is then [T, Hq * value_dim].  ``head_scales`` (float32
+    [Hq]): every head's scores are multiplied by its number (after ``scale``).  ``sigmoid``: a visible key weighs
+    sigmoid(score + ``score_bias[head]``) (float32 [Hq] or None) on its own and nothing is normalized."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -954,6 +995,11 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
           "paged_attention: log_bias must be float32 [Hq, 2] on the GPU")
     _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads and sinks.is_contiguous()
                             and sinks.is_cuda), "paged_attention: sinks must be float32 [Hq] on the GPU")
+    for name, one in (("head_scales", head_scales), ("score_bias", score_bias)):
+        _need(one is None or (one.dtype == torch.float32 and one.numel() == num_heads and one.is_contiguous()
+                              and one.is_cuda), f"paged_attention: {name} must be float32 [Hq] on the GPU")
+    _need(sigmoid or score_bias is None, "paged_attention: a bias per head is for sigmoid weights")
+    _need(not (sigmoid and sinks is not None), "paged_attention: a sink belongs to a softmax")
     holds = block_tables.shape[1] * page_size
     span = holds if max_seq_len is None else max(1, min(int(max_seq_len), holds))
     floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, value_dim, span)
@@ -970,7 +1016,58 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
         int(window or 0), _p(slopes), _p(log_bias), _p(sinks), span, _p(partial), partial.numel(), _p(out), out_ld,
         _p(query_tiles) if tiles else None, tiles, int(tile_tokens) if tiles else 0, _p(cu_seqlens) if tiles else None,
-        _stream()), "paged_attention", f"(head_dim={head_dim})")
+        _p(head_scales), _p(score_bias), 1 if sigmoid else 0, _stream()), "paged_attention", f"(head_dim={head_dim})")
+
+
+def attention_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                      positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rotary_dim: int,
+                      slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                      v_cache: Optional[torch.Tensor], *, values_from_keys: bool = False,
+                      q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+                      norm_eps: float = 0.0, value_inv_freq: Optional[torch.Tensor] = None) -> None:
+    """A token's projected row made ready for attention, one launch: ``qkv`` [T, >= Hq*dh + Hkv*dh (+ Hkv*dv)]
+    holds q heads, k heads and (unless ``values_from_keys``) v heads.
+
+    * ``q_norm`` / ``k_norm`` (float32 [Hq*dh] / [Hkv*dh]): the whole q projection, and the whole k projection, is
+      divided by its root mean square (``norm_eps`` inside the root) and multiplied by the weight, before rotation;
+    * q and k are turned by the token's position (half-split pairs over the first ``rotary_dim`` dims, angle =
+      position * inv_freq[j]); q is written back in place, k goes to the token's cache cell;
+    * the values are the v heads, or with ``values_from_keys`` the k heads as projected (before norm and rotation);
+      with ``value_inv_freq`` (float32 [dv / 2]) they are turned by the position over all their dims (half-split
+      pairs); they go to the token's (transposed) cache cell.
+
+    Norms, angles and rotations are float32.  Without ``slot_mapping`` nothing is stored."""
+    ld = _row_major(qkv, "qkv")
+    T = qkv.shape[0]
+    value_dim = int(value_dim)
+    q_cols, k_cols = num_heads * head_dim, num_kv_heads * head_dim
+    v_cols = 0 if values_from_keys else num_kv_heads * value_dim
+    _need(qkv.shape[1] >= q_cols + k_cols + v_cols, "attention_prepare: qkv is too narrow")
+    _need(not values_from_keys or value_dim == head_dim, "attention_prepare: values that are the keys have their width")
+    _i32(positions, "positions")
+    _need(positions.numel() == T, "attention_prepare: one position per token")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2 and inv_freq.is_cuda
+              and 0 < rotary_dim <= head_dim and rotary_dim % 2 == 0,
+              "attention_prepare: inv_freq must be float32 [rotary_dim / 2]")
+    if value_inv_freq is not None:
+        _need(value_inv_freq.dtype == torch.float32 and value_dim % 2 == 0 and value_inv_freq.numel() == value_dim // 2
+              and value_inv_freq.is_cuda, "attention_prepare: value_inv_freq must be float32 [value_dim / 2]")
+    _need((q_norm is None) == (k_norm is None), "attention_prepare: both projections are normed or neither")
+    if q_norm is not None:
+        _need(q_norm.dtype == torch.float32 and q_norm.numel() == q_cols and q_norm.is_contiguous() and q_norm.is_cuda
+              and k_norm.dtype == torch.float32 and k_norm.numel() == k_cols and k_norm.is_contiguous()
+              and k_norm.is_cuda and norm_eps > 0, "attention_prepare: the norms' weights must be float32 [Hq*dh], [Hkv*dh]")
+    page_stride, page_size = 0, 0
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "attention_prepare: one cache cell per token")
+        page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, value_dim)
+    _check(_fn("attention", "mi_attention_prepare")(
+        _p(qkv), _dt(qkv), ld, T, num_heads, num_kv_heads, head_dim, value_dim, 1 if values_from_keys else 0,
+        _p(positions), _p(inv_freq), int(rotary_dim) if inv_freq is not None else 0, _p(q_norm), _p(k_norm),
+        float(norm_eps), _p(value_inv_freq), _p(slot_mapping), _p(k_cache) if slot_mapping is not None else None,
+        _p(v_cache) if slot_mapping is not None else None, page_stride, page_size, _stream()), "attention_prepare")
 
 
 def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:

@@ -9,6 +9,7 @@ from ..kernels.limits import ATTENTION_MAX_HEAD_DIM, GRID_MOST, beyond
 from ..weights.loader import Expect
 from .base import BuildContext, Mixer, part_class, register_part
 from .linear import Linear
+from .position import rotary_frequencies
 
 
 @register_part("attention")
@@ -23,6 +24,12 @@ class Attention(Mixer):
     per query head whose exponential is one more term of the denominator, with no key and no value), and the
     position encoding may be a bias on the scores; all three take the general attention kernel.
 
+    Further forms, each a field of the spec: values that are the keys as projected (no v projection); an RMS norm
+    over the whole q and the whole k projection before rotation; values turned by their position before they are
+    cached and outputs turned back by the query's; a learned multiplier of every head's scores; sigmoid weights
+    with a learned bias per head in place of the softmax.  One kernel prepares a token's row for all of them
+    (``ops.attention_prepare``: norms, rotations, cache write).
+
     Multipliers: ``in_multiplier`` scales the input of q/k/v (folded into their weights),
     ``key_multiplier`` the k projection's output (weights and bias), ``out_multiplier``
     the output projection's output."""
@@ -36,17 +43,26 @@ class Attention(Mixer):
         kv_rows = spec.num_kv_heads * spec.head_dim
         v_rows = spec.num_kv_heads * spec.value_width
         out = [Expect(f"{prefix}.q_proj.weight", ((q_rows, hidden_size),)),
-               Expect(f"{prefix}.k_proj.weight", ((kv_rows, hidden_size),)),
-               Expect(f"{prefix}.v_proj.weight", ((v_rows, hidden_size),)),
-               Expect(f"{prefix}.o_proj.weight", ((hidden_size, spec.num_heads * spec.value_width),))]
+               Expect(f"{prefix}.k_proj.weight", ((kv_rows, hidden_size),))]
+        if not spec.values_from_keys:
+            out.append(Expect(f"{prefix}.v_proj.weight", ((v_rows, hidden_size),)))
+        out.append(Expect(f"{prefix}.o_proj.weight", ((hidden_size, spec.num_heads * spec.value_width),)))
         if spec.qkv_bias:
             out += [Expect(f"{prefix}.q_proj.bias", ((q_rows,),), init="bias"),
-                    Expect(f"{prefix}.k_proj.bias", ((kv_rows,),), init="bias"),
-                    Expect(f"{prefix}.v_proj.bias", ((v_rows,),), init="bias")]
+                    Expect(f"{prefix}.k_proj.bias", ((kv_rows,),), init="bias")]
+            if not spec.values_from_keys:
+                out.append(Expect(f"{prefix}.v_proj.bias", ((v_rows,),), init="bias"))
         if spec.out_bias:
             out.append(Expect(f"{prefix}.o_proj.bias", ((hidden_size,),), init="bias"))
         if spec.sink:
             out.append(Expect(f"{prefix}.sink", ((spec.num_heads,),), init="logit"))
+        if spec.projection_norm_eps is not None:
+            out += [Expect(f"{prefix}.q_norm.weight", ((q_rows,),), init="norm"),
+                    Expect(f"{prefix}.k_norm.weight", ((kv_rows,),), init="norm")]
+        if spec.head_temperature:
+            out.append(Expect(f"{prefix}.temp", ((spec.num_heads,),), init="positive"))
+        if spec.score_bias:
+            out.append(Expect(f"{prefix}.pb", ((spec.num_heads,),), init="logit"))
         out += part_class(spec.position).expected_tensors(spec.position, prefix, hidden_size)
         return out
 
@@ -69,13 +85,15 @@ class Attention(Mixer):
         kv_rows = spec.num_kv_heads * spec.head_dim
         v_rows = spec.num_kv_heads * spec.value_width
         get = lambda name: tensors.get(f"{prefix}.{name}")
+        if spec.values_from_keys:
+            v_rows = 0
         weight_scale = torch.cat([torch.full((q_rows,), spec.in_multiplier),
                                   torch.full((kv_rows,), spec.in_multiplier * spec.key_multiplier),
                                   torch.full((v_rows,), spec.in_multiplier)])
         bias_scale = torch.cat([torch.ones(q_rows), torch.full((kv_rows,), spec.key_multiplier),
                                 torch.ones(v_rows)])
-        self.qkv = Linear([get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")],
-                          [get("q_proj.bias"), get("k_proj.bias"), get("v_proj.bias")], build,
+        names = ("q_proj", "k_proj") if spec.values_from_keys else ("q_proj", "k_proj", "v_proj")
+        self.qkv = Linear([get(f"{name}.weight") for name in names], [get(f"{name}.bias") for name in names], build,
                           weight_scale=weight_scale, bias_scale=bias_scale)
         self.out = Linear([get("o_proj.weight")], [get("o_proj.bias")], build,
                           weight_scale=spec.out_multiplier, bias_scale=spec.out_multiplier)
@@ -84,11 +102,31 @@ class Attention(Mixer):
             self.position = position_class(spec.position, spec.head_dim, build, prefix=prefix, tensors=tensors)
         else:
             self.position = position_class(spec.position, spec.head_dim, build)
-        self.sink = get("sink").to(torch.float32).contiguous().to(build.device) if spec.sink else None
+        f32 = lambda name: get(name).to(torch.float32).contiguous().to(build.device)
+        self.sink = f32("sink") if spec.sink else None
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))
+        # the forms that ``ops.attention_prepare`` and the general kernel's extra terms serve
+        self.head_scales = f32("temp") if spec.head_temperature else None
+        self.score_bias = f32("pb") if spec.score_bias else None
+        self.q_norm = f32("q_norm.weight") if spec.projection_norm_eps is not None else None
+        self.k_norm = f32("k_norm.weight") if spec.projection_norm_eps is not None else None
+        self.value_inv_freq = None
+        if spec.value_rotation_theta is not None:
+            turns = rotary_frequencies(spec.value_rotation_theta, spec.value_width)
+            self.value_inv_freq = torch.tensor(turns, dtype=torch.float64).to(torch.float32).to(build.device)
+            self.value_inv_freq_back = (-self.value_inv_freq).contiguous()
+        self.prepared = (spec.values_from_keys or spec.projection_norm_eps is not None
+                         or spec.value_rotation_theta is not None or spec.head_temperature
+                         or spec.weighting != "softmax")
+        if self.prepared:
+            rotation = self.position.fused_rotation()
+            if rotation is None or self.position.score_slopes is not None or self.position.score_log_bias is not None:
+                raise ValueError(f"{prefix}: this form of attention turns q and k itself: the position encoding "
+                                 f"{spec.position.kind!r} is no rotation by position")
+            self.inv_freq, self.rotary_dim = rotation
         # what only the general kernel knows: a bias on the scores, a sink, values of another width than the keys
         self.general_only = (self.position.score_slopes is not None or self.position.score_log_bias is not None
-                             or self.sink is not None or spec.value_width != spec.head_dim)
+                             or self.sink is not None or spec.value_width != spec.head_dim or self.prepared)
 
     def projections(self):
         if self.general_only:          # the fused decode kernels know none of it: the layer runs part by part
@@ -107,6 +145,9 @@ class Attention(Mixer):
         spec = self.spec
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
         slopes = self.position.score_slopes
+        if self.prepared:
+            self.mix_prepared(qkv, step, cache, attended)
+            return
         if self.general_only:
             self.position.rotate(qkv, *geometry, step)
             if cache.owns_kv:
@@ -153,3 +194,47 @@ class Attention(Mixer):
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended,
                                 step.max_seq_len, **tiles)
+
+    def mix_prepared(self, qkv: torch.Tensor, step, cache, attended: torch.Tensor) -> None:
+        """The forms that go through ``ops.attention_prepare``: one launch norms the q and k projections, turns q
+        (in place) and k, turns the values or takes the keys as projected for them, and writes the token's cache
+        cells; the attention kernels then see ordinary cached keys and values."""
+        spec = self.spec
+        geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
+        owns = cache.owns_kv
+        ops.attention_prepare(qkv, *geometry, spec.value_width, step.positions, self.inv_freq, self.rotary_dim,
+                              step.slot_mappings[cache.group] if owns else None, cache.k_cache if owns else None,
+                              cache.v_cache if owns else None, values_from_keys=spec.values_from_keys,
+                              q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=spec.projection_norm_eps or 0.0,
+                              value_inv_freq=self.value_inv_freq)
+        target = attended
+        if self.value_inv_freq is not None:         # the heads' outputs are turned back into ``attended`` below
+            target = torch.empty((qkv.shape[0], spec.num_heads * spec.value_width), dtype=qkv.dtype, device=qkv.device)
+        self.attend_prepared(qkv, step, cache, target)
+        if target is not attended:
+            ops.rotate_heads(target, 0, spec.value_width, spec.num_heads, spec.value_width, step.positions,
+                             self.value_inv_freq_back, spec.value_width, False, attended, 0, spec.value_width)
+
+    def attend_prepared(self, qkv: torch.Tensor, step, cache, out: torch.Tensor) -> None:
+        spec = self.spec
+        geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
+        sigmoid = spec.weighting == "sigmoid"
+        tiles = {}
+        if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
+            tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
+        plain = not sigmoid and self.head_scales is None and spec.value_width == spec.head_dim
+        aligned = (qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 and out.stride(0) % 4 == 0
+                   and out.data_ptr() % 8 == 0)
+        if plain and step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
+            ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                 step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len, out)
+        elif (plain and tiles and aligned and step.query_tile == self.query_tile
+                and ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2])):
+            ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                  step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window, out,
+                                  step.max_seq_len)
+        else:
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, out, step.max_seq_len,
+                                value_dim=spec.value_width, head_scales=self.head_scales, score_bias=self.score_bias,
+                                sigmoid=sigmoid, **tiles)

@@ -94,9 +94,20 @@ class RowVector:
     vector: torch.Tensor
 
 
+@dataclass
+class NormedBranches:
+    """Branch outputs whose weighted sum goes through a layer norm of its own before it joins the residual stream:
+    x <- x + ((s - mean) / sqrt(variance + eps) * weight + bias) with s = sum of factor * rows over ``branches``
+    [(rows [T, d], factor)], everything in float32."""
+    branches: list
+    weight: torch.Tensor
+    bias: torch.Tensor
+    eps: float
+
+
 class Residual:
     """The float32 residual stream [T, d] plus the branch outputs not yet added to it (tensors,
-    ``ScaledBranch``es, ``WeightedBranch``es or ``RowVector``s).  The next norm adds them and normalizes in one kernel.
+    ``ScaledBranch``es, ``WeightedBranch``es, ``NormedBranches`` or ``RowVector``s).  The next norm adds them and normalizes in one kernel.
 
     ``next_norm``: (weight, eps) of the norm that the layer after the one running starts with (the final norm
     after the last), if that norm is a root-mean-square norm, set by whoever runs the layers; a layer whose last

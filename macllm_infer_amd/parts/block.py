@@ -6,7 +6,7 @@ from typing import Dict
 import torch
 
 from ..weights.loader import Expect
-from .base import BuildContext, Residual, ScaledBranch, WeightedBranch, part_class
+from .base import BuildContext, NormedBranches, Residual, ScaledBranch, WeightedBranch, part_class
 
 _ARRANGEMENTS: Dict[str, type] = {}
 _FUSIONS: Dict[str, object] = {}
@@ -132,8 +132,9 @@ class ParallelPreNormBlock:
         factory = _FUSIONS.get(layer.arrangement)
         # the fast path knows plain branches and a feed-forward behind them; None when parts or sizes do not fit
         self.branch_multiplier = float(getattr(layer, "branch_multiplier", 1.0))
+        self.mixer_weights = [float(getattr(slot, "weight", 1.0)) for slot in layer.mixers]
         plain = (self.mixer_scale is None and self.ffn_scale is None and self.ffn is not None
-                 and self.branch_multiplier == 1.0)
+                 and self.branch_multiplier == 1.0 and all(weight == 1.0 for weight in self.mixer_weights))
         self.fusion = factory(self, build) if factory is not None and plain else None
 
     @property
@@ -160,24 +161,12 @@ class ParallelPreNormBlock:
         if fusion is not None and fusion.forward(residual, step, caches):
             return
         normed = self.mixer_norm.forward(residual)
-        if overlap_pays([mixer for _, mixer in self.mixers], normed.shape[0], normed.device):
-            # the second mixer is recorded first and stays on the queue of the kernels around it (see the fast
-            # path's ``forward_general``); what either allocates is its own stream's until the join
-            (first_name, first), (second_name, second) = self.mixers
-            main = torch.cuda.current_stream(normed.device)
-            side = side_stream(normed.device, main)
-            side.wait_stream(main)
-            second_out = second.forward(normed, step, caches[second_name])
-            with torch.cuda.stream(side):
-                first_out = first.forward(normed, step, caches[first_name])
-            main.wait_stream(side)
-            outputs = [first_out, second_out]
-        else:
-            outputs = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+        outputs = self.run_mixers(normed, step, caches)
         if self.mixer_scale is not None:
             outputs = [ScaledBranch(rows, self.mixer_scale) for rows in outputs]
-        elif self.branch_multiplier != 1.0:
-            outputs = [WeightedBranch(rows, self.branch_multiplier) for rows in outputs]
+        elif self.branch_multiplier != 1.0 or any(weight != 1.0 for weight in self.mixer_weights):
+            outputs = [WeightedBranch(rows, self.branch_multiplier * weight)
+                       for rows, weight in zip(outputs, self.mixer_weights)]
         residual.pending = outputs
         if self.ffn is None:
             return
@@ -189,3 +178,64 @@ class ParallelPreNormBlock:
             residual.pending = [WeightedBranch(rows, self.branch_multiplier)]
         else:
             residual.pending = [rows]
+
+    def run_mixers(self, normed: torch.Tensor, step, caches) -> list:
+        """Every mixer's output for the normed rows, in the mixers' order."""
+        if overlap_pays([mixer for _, mixer in self.mixers], normed.shape[0], normed.device):
+            # the second mixer is recorded first and stays on the queue of the kernels around it (see the fast
+            # path's ``forward_general``); what either allocates is its own stream's until the join
+            (first_name, first), (second_name, second) = self.mixers
+            main = torch.cuda.current_stream(normed.device)
+            side = side_stream(normed.device, main)
+            side.wait_stream(main)
+            second_out = second.forward(normed, step, caches[second_name])
+            with torch.cuda.stream(side):
+                first_out = first.forward(normed, step, caches[first_name])
+            main.wait_stream(side)
+            return [first_out, second_out]
+        return [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+
+
+@register_arrangement("sandwich")
+class SandwichBlock(ParallelPreNormBlock):
+    """A norm before and a norm after each branch: h += post1(sum over mixers of weight_m * mixer_m(norm1(h)));
+    h += post2(ffn(norm2(h))).  The weighted sum of a branch and its post-norm wait in ``Residual.pending`` as one
+    ``NormedBranches`` entry, so the norm that follows (this layer's second, or the next layer's first) takes the
+    branch through its post-norm, adds it to the stream and normalizes the stream in one launch."""
+
+    @classmethod
+    def expected_tensors(cls, layer, hidden_size: int):
+        out = super().expected_tensors(layer, hidden_size)
+        post = part_class(layer.mixer_post_norm).expected_tensors(
+            layer.mixer_post_norm, f"{layer.prefix}.{layer.mixer_post_norm_name}", hidden_size)
+        second = part_class(layer.ffn_post_norm).expected_tensors(
+            layer.ffn_post_norm, f"{layer.prefix}.{layer.ffn_post_norm_name}", hidden_size)
+        if layer.ffn is None:
+            second = [Expect(one.name, one.shapes, one.init, one.integer, optional=True) for one in second]
+        return out + post + second
+
+    @staticmethod
+    def _part_specs(layer):
+        return ParallelPreNormBlock._part_specs(layer) + [layer.mixer_post_norm]
+
+    def __init__(self, layer, tensors, build: BuildContext):
+        super().__init__(layer, tensors, build)
+        self.fusion = None
+        if layer.mixer_post_norm.kind != "layernorm" or (layer.ffn is not None and layer.ffn_post_norm.kind != "layernorm"):
+            raise ValueError(f"layer {layer.prefix}: the norms behind the branches of a sandwich layer are layer norms")
+
+        def post(spec, name):
+            norm = part_class(spec)(spec, f"{layer.prefix}.{name}", tensors, build)
+            return norm.weight, norm.bias, float(spec.eps)
+        self.mixer_post = post(layer.mixer_post_norm, layer.mixer_post_norm_name)
+        self.ffn_post = post(layer.ffn_post_norm, layer.ffn_post_norm_name) if layer.ffn is not None else None
+
+    def forward(self, residual: Residual, step, caches) -> None:
+        normed = self.mixer_norm.forward(residual)
+        outputs = self.run_mixers(normed, step, caches)
+        branches = [(rows, self.branch_multiplier * weight) for rows, weight in zip(outputs, self.mixer_weights)]
+        residual.pending = [NormedBranches(branches, *self.mixer_post)]
+        if self.ffn is None:
+            return
+        normed = self.ffn_norm.forward(residual)
+        residual.pending = [NormedBranches([(self.ffn.forward(normed), self.branch_multiplier)], *self.ffn_post)]

@@ -11,8 +11,8 @@ from .linear import Linear
 
 @register_part("swiglu")
 class SwiGLU(FeedForward):
-    """down(SiLU(gate(x)) * up(x)); gate and up are one fused product
-    (reference: src/decoder.rs:261-306).  ``gate_multiplier`` scales gate's output,
+    """down(act(gate(x)) * up(x)), act = SiLU or the tanh form of GELU (``activation``); gate and up are one fused
+    product (reference: src/decoder.rs:261-306).  ``gate_multiplier`` scales gate's output,
     ``down_multiplier`` down's output; both are folded into the weights.  When the width is a
     multiple of 8 the rows of the fused matrix are stored in tiles of 8 gate rows and 8 up rows
     (``tile``), the order the fused decode kernel wants, so that one matrix serves every path."""
@@ -49,12 +49,14 @@ class SwiGLU(FeedForward):
                 self.gate_up.bias = self.gate_up.bias[order].contiguous()
 
     def gated_projections(self):
+        if self.spec.activation != "silu":          # the fused decode kernels apply SiLU
+            return None
         return self.gate_up, self.down, self.tile
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         gate_up = self.gate_up(x)
         activated = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=gate_up.dtype, device=x.device)
-        ops.swiglu(gate_up, activated, self.tile)
+        ops.swiglu(gate_up, activated, self.tile, activation=self.spec.activation)
         return self.down(activated)
 
 

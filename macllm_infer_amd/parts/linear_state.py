@@ -160,3 +160,73 @@ class GeneralDelta(Mixer):
         ops.head_norm_gate(raw, u[:, 3 * inner:4 * inner], self.norm_weight, spec.num_heads, spec.norm_eps, "sigmoid",
                            gated)
         return self.out_proj(gated)
+
+
+@register_part("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    """[q | k | v | g | a1] = one projection of the normed rows; decay logits z = a2 (a1 part) in float32; inside the
+    scan q is multiplied by ``query_scale`` and alpha = sigmoid(z + bias)^(1 / temperature) = exp(log sigmoid / temperature)
+    decays every key channel of the state on its own, S <- diag(alpha) S + k v^T, o = S^T q; then o / rms(o) per head
+    times a weight of value_dim numbers that the heads share, times SiLU(g), output projection."""
+    graph_safe = True
+    kernel_modules = ("common", "linear_state", "gemm")
+    chunk_tokens = CHUNK_TOKENS
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        keys, values = spec.num_heads * spec.key_dim, spec.num_heads * spec.value_dim
+        rank = -1 if spec.decay_rank is None else spec.decay_rank
+        return [Expect(f"{prefix}.q.weight", ((keys, hidden_size),)),
+                Expect(f"{prefix}.k.weight", ((keys, hidden_size),)),
+                Expect(f"{prefix}.v.weight", ((values, hidden_size),)),
+                Expect(f"{prefix}.g.weight", ((values, hidden_size),)),
+                Expect(f"{prefix}.a1.weight", ((rank, hidden_size),)),
+                Expect(f"{prefix}.a2.weight", ((keys, rank),)),
+                Expect(f"{prefix}.a2.bias", ((keys,),), init="logit"),
+                Expect(f"{prefix}.norm.weight", ((spec.value_dim,),), init="norm"),
+                Expect(f"{prefix}.o.weight", ((hidden_size, values),))]
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        return (beyond("gated_linear_attention", "key_dim", spec.key_dim, LINEAR_STATE_MAX_KEY_DIM,
+                       "a column of a head's state is spread over at most one wave")
+                + beyond("gated_linear_attention", "num_heads", spec.num_heads, GRID_MOST,
+                         "heads index a dimension of the launch"))
+
+    @classmethod
+    def cache_needs(cls, spec):
+        return [StateNeed("state", (spec.num_heads, spec.value_dim, spec.key_dim), "float32")]
+
+    def __init__(self, spec, prefix: str, tensors, build: BuildContext):
+        self.spec = spec
+        get = lambda name: tensors.get(f"{prefix}.{name}")
+        if get("a1.weight").shape[0] != get("a2.weight").shape[1]:
+            raise ValueError(f"{prefix}: the decay's two projections do not fit each other: "
+                             f"{tuple(get('a1.weight').shape)} and {tuple(get('a2.weight').shape)}")
+        self.rank = get("a1.weight").shape[0]
+        self.in_proj = Linear([get("q.weight"), get("k.weight"), get("v.weight"), get("g.weight"), get("a1.weight")],
+                              [None, None, None, None, None], build)
+        self.decay_proj = Linear([get("a2.weight")], [None], build)
+        self.out_proj = Linear([get("o.weight")], [None], build)
+        f32 = lambda tensor: tensor.to(torch.float32).contiguous().to(build.device)
+        self.decay_bias = f32(get("a2.bias"))
+        self.norm_weight = f32(get("norm.weight")).repeat(spec.num_heads).contiguous()      # one copy a head
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        spec = self.spec
+        keys, values = spec.num_heads * spec.key_dim, spec.num_heads * spec.value_dim
+        u = self.in_proj(x)                                              # [T, q | k | v | g | a1]
+        inner = u[:, 2 * keys + 2 * values:]
+        if inner.stride(0) % 8 != 0 or inner.data_ptr() % 16 != 0:      # the product wants whole 16-byte pieces
+            inner = inner.contiguous()
+        logits = ops.linear(inner, self.decay_proj.weight, None, keep_float32=True)      # float32 [T, H * dk]
+        raw = torch.empty((x.shape[0], values), dtype=torch.float32, device=x.device)
+        ops.linear_state_scan(u, q_col=0, k_col=keys, v_col=2 * keys, num_heads=spec.num_heads, key_dim=spec.key_dim,
+                              value_dim=spec.value_dim, state=cache.states["state"], cu_seqlens=step.cu_seqlens,
+                              slot_ids=step.slot_ids, out=raw, max_query_len=step.max_query_len,
+                              decay_logits=logits, decay_bias=self.decay_bias, gate_power=1.0 / spec.decay_temperature,
+                              query_scale=spec.query_scale, chunks=scan_chunks(step))
+        gated = torch.empty((x.shape[0], values), dtype=u.dtype, device=x.device)
+        ops.head_norm_gate(raw, u[:, 2 * keys + values:2 * keys + 2 * values], self.norm_weight, spec.num_heads,
+                           spec.norm_eps, "silu", gated)
+        return self.out_proj(gated)

@@ -8,7 +8,7 @@ import torch
 from ..kernels import ops
 from ..kernels.limits import NORM_MAX_WIDTH, beyond
 from ..weights.loader import Expect
-from .base import BuildContext, Part, Residual, RowVector, ScaledBranch, WeightedBranch, register_part
+from .base import BuildContext, NormedBranches, Part, Residual, RowVector, ScaledBranch, WeightedBranch, register_part
 
 
 def partial_slab(pending) -> Optional[torch.Tensor]:
@@ -26,12 +26,31 @@ def partial_slab(pending) -> Optional[torch.Tensor]:
     return base
 
 
+def add_normed_branches(h: torch.Tensor, normed: NormedBranches, vector: Optional[torch.Tensor] = None) -> None:
+    """h += layer norm of the weighted sum of ``normed``'s branches (+ ``vector`` on every row); nothing is normed
+    behind it."""
+    branches = list(normed.branches)
+    extra = None
+    while len(branches) > LAYERNORM_BRANCHES:               # more than the kernel sums: the first ones are added up first
+        first, factor = branches.pop(0)
+        if extra is None:
+            extra = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+        ops.stream_add(extra, first, factor, None)
+    if extra is not None:
+        second, factor = branches.pop(0)
+        ops.stream_add(extra, second, factor, None)
+        branches.insert(0, (extra, 1.0))
+    ops.add_layernorm(h, branches, vector, None, None, 0.0, None, branch_norm=(normed.weight, normed.bias, normed.eps))
+
+
 def fold_weighted(residual: Residual) -> None:
-    """Add the ``WeightedBranch``es and ``RowVector``s among the pending branches to the stream with the kernel
-    that knows them, and leave the others pending: for a norm whose own kernel fuses neither."""
+    """Add the ``WeightedBranch``es, ``NormedBranches`` and ``RowVector``s among the pending branches to the stream
+    with the kernel that knows them, and leave the others pending: for a norm whose own kernel fuses none of them."""
     kept = []
     for branch in residual.pending:
-        if isinstance(branch, WeightedBranch):
+        if isinstance(branch, NormedBranches):
+            add_normed_branches(residual.h, branch)
+        elif isinstance(branch, WeightedBranch):
             ops.stream_add(residual.h, branch.rows, branch.factor, None)
         elif isinstance(branch, RowVector):
             ops.stream_add(residual.h, None, 1.0, branch.vector)
@@ -39,6 +58,16 @@ def fold_weighted(residual: Residual) -> None:
             kept.append(branch)
     if len(kept) != len(residual.pending):
         residual.pending = kept
+
+
+def fold_pending(residual: Residual) -> None:
+    """Add everything that is pending to the stream, with no norm behind it."""
+    fold_weighted(residual)
+    for branch in residual.pending:
+        if isinstance(branch, ScaledBranch):
+            raise NotImplementedError("a branch scaled by feature joins the stream in a norm's kernel")
+        ops.stream_add(residual.h, branch, 1.0, None)
+    residual.pending = []
 
 
 @register_part("rmsnorm")
@@ -74,7 +103,7 @@ class RmsNorm(Part):
     def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add the pending branch outputs to the residual stream and return its normed rows
         (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""
-        if any(isinstance(branch, (WeightedBranch, RowVector)) for branch in residual.pending):
+        if any(isinstance(branch, (WeightedBranch, RowVector, NormedBranches)) for branch in residual.pending):
             fold_weighted(residual)
         pending = residual.pending
         slab = partial_slab(pending)
@@ -142,9 +171,15 @@ class LayerNorm(Part):
     def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add the pending branches to the stream and return its normed rows (all, or only ``rows``; with ``rows``
         the stream itself is left unchanged and the branches stay pending)."""
-        branches, vector = [], None
+        branches, vector, normed = [], None, None
         for branch in residual.pending:
-            if isinstance(branch, RowVector):
+            if isinstance(branch, NormedBranches):
+                # the one the kernel takes through its own norm on the way into the stream; others before it
+                if normed is not None or rows is not None or len(branch.branches) > LAYERNORM_BRANCHES:
+                    add_normed_branches(residual.h, branch)
+                else:
+                    normed = branch
+            elif isinstance(branch, RowVector):
                 if vector is None:
                     vector = branch.vector
                 else:                                      # a second vector: added by the plain kernel
@@ -155,11 +190,21 @@ class LayerNorm(Part):
                 branches.append((branch.rows, float(branch.factor)))
             else:
                 branches.append((branch, 1.0))
+        if normed is not None and branches:
+            # plain branches beside a normed group: the plain ones go first, the kernel's branch slots are the group's
+            for tensor, factor in branches:
+                ops.stream_add(residual.h, tensor, factor, None)
+            branches = []
         while len(branches) > LAYERNORM_BRANCHES:
             first, factor = branches.pop(0)
             ops.stream_add(residual.h, first, factor, None)
         count = residual.h.shape[0] if rows is None else rows.numel()
         out = torch.empty((count, residual.h.shape[1]), dtype=self.build.dtype, device=residual.h.device)
+        if normed is not None:
+            ops.add_layernorm(residual.h, normed.branches, vector, self.weight, self.bias, self.eps, out,
+                              branch_norm=(normed.weight, normed.bias, normed.eps))
+            residual.pending = []
+            return out
         ops.add_layernorm(residual.h, branches, vector, self.weight, self.bias, self.eps, out, rows)
         if rows is None:
             residual.pending = []

@@ -65,16 +65,37 @@ class NoPosition(PositionEncoding):
         return None, 0, False
 
 
+def rotary_frequencies(theta: float, rotary_dim: int, scaling=None) -> list:
+    """f_j = theta^(-2j / rotary_dim), j below rotary_dim / 2, in float64; with ``scaling`` (factor, low, high,
+    original) stretched by wavelength l = 2 pi / f: kept where l < original / high, f / factor where
+    l > original / low, between the two (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    import math
+    frequencies = [1.0 / (theta ** (index / rotary_dim)) for index in range(0, rotary_dim, 2)]
+    if scaling is None:
+        return frequencies
+    out = []
+    for frequency in frequencies:
+        wavelength = 2.0 * math.pi / frequency
+        if wavelength < scaling.original / scaling.high:
+            out.append(frequency)
+        elif wavelength > scaling.original / scaling.low:
+            out.append(frequency / scaling.factor)
+        else:
+            blend = (scaling.original / wavelength - scaling.low) / (scaling.high - scaling.low)
+            out.append((1.0 - blend) * frequency / scaling.factor + blend * frequency)
+    return out
+
+
 @register_part("rope")
 class Rope(PositionEncoding):
-    """Half-split rotary encoding: f_j = theta^(-2j/rotary_dim) formed in float64 and rounded
-    to float32; angle = position * f_j, cos and sin in float32
+    """Half-split rotary encoding: f_j = theta^(-2j/rotary_dim) formed in float64 (stretched by wavelength when the
+    spec says so) and rounded to float32; angle = position * f_j, cos and sin in float32
     (reference: src/decoder.rs:136-144, 186-195, 226-229)."""
     graph_safe = True
 
     def __init__(self, spec, head_dim: int, build: BuildContext):
         self.rotary_dim = spec.rotary_dim
-        frequencies = [1.0 / (spec.theta ** (index / spec.rotary_dim)) for index in range(0, spec.rotary_dim, 2)]
+        frequencies = rotary_frequencies(spec.theta, spec.rotary_dim, getattr(spec, "scaling", None))
         self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
 
     def fused_rotation(self):

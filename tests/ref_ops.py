@@ -40,14 +40,60 @@ def add_rmsnorm(h, deltas, weight, eps, out, rows=None):
         out.copy_(normed.to(out.dtype))
 
 
-def swiglu(gate_up, out, tile=0):
+def cast_rows(source, out):
+    out.copy_(source.to(out.dtype))
+
+
+def attention_prepare(qkv, num_heads, num_kv_heads, head_dim, value_dim, positions, inv_freq, rotary_dim, slot_mapping,
+                      k_cache, v_cache, *, values_from_keys=False, q_norm=None, k_norm=None, norm_eps=0.0,
+                      value_inv_freq=None):
+    T = qkv.shape[0]
+    q_cols, k_cols = num_heads * head_dim, num_kv_heads * head_dim
+    q = _f(qkv[:, :q_cols]).clone()
+    k = _f(qkv[:, q_cols:q_cols + k_cols]).clone()
+    if values_from_keys:
+        v = k.clone().reshape(T, num_kv_heads, head_dim)
+    else:
+        v = _f(qkv[:, q_cols + k_cols:q_cols + k_cols + num_kv_heads * value_dim]).reshape(T, num_kv_heads, value_dim).clone()
+    if q_norm is not None:
+        q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + norm_eps) * q_norm
+        k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + norm_eps) * k_norm
+    q = q.reshape(T, num_heads, head_dim)
+    k = k.reshape(T, num_kv_heads, head_dim)
+    spots = positions.to(torch.float32)
+
+    def rotate(x, frequencies, width):
+        half = width // 2
+        angle = spots[:, None] * frequencies[None, :]
+        cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+        a, b = x[..., :half], x[..., half:width]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., width:]], dim=-1)
+    if inv_freq is not None and rotary_dim > 0:
+        q, k = rotate(q, inv_freq, rotary_dim), rotate(k, inv_freq, rotary_dim)
+    if value_inv_freq is not None:
+        v = rotate(v, value_inv_freq, value_dim)
+    qkv[:, :q_cols] = q.reshape(T, q_cols).to(qkv.dtype)
+    if slot_mapping is not None:
+        page_size = k_cache.shape[2]
+        pages = (slot_mapping // page_size).long()
+        offsets = (slot_mapping % page_size).long()
+        k_cache[pages, :, offsets, :] = k.to(k_cache.dtype)
+        v_cache[pages, :, :, offsets] = v.to(v_cache.dtype)
+
+
+def swiglu(gate_up, out, tile=0, activation="silu"):
     inner = gate_up.shape[1] // 2
     if tile:
         tiles = gate_up.reshape(gate_up.shape[0], inner // tile, 2, tile)
         gate, up = tiles[:, :, 0].reshape(-1, inner), tiles[:, :, 1].reshape(-1, inner)
     else:
         gate, up = gate_up[:, :inner], gate_up[:, inner:]
-    out.copy_((F.silu(_f(gate)) * _f(up)).to(out.dtype))
+    if activation == "gelu_tanh":
+        z = _f(gate)
+        bent = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+    else:
+        bent = F.silu(_f(gate))
+    out.copy_((bent * _f(up)).to(out.dtype))
 
 
 def scale_to_f32(values, multiplier, out):
@@ -113,7 +159,8 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
                     positions, scale, window, out, max_seq_len=None, slopes=None, query_tiles=None, tile_tokens=0,
-                    cu_seqlens=None, log_bias=None, sinks=None, value_dim=None):
+                    cu_seqlens=None, log_bias=None, sinks=None, value_dim=None, head_scales=None, score_bias=None,
+                    sigmoid=False):
     """``max_seq_len`` sizes the kernel's launch and nothing else: not used here, and neither is the table of
     runs that picks the kernel for lanes of several tokens.  ``slopes``: a bias on the scores,
     ``-slopes[head] * (query position - key position)``; ``log_bias`` [Hq, 2] = (r1, r2): the scores lose
@@ -134,6 +181,12 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
         for head in range(num_heads):
             query = _f(q[token, head * head_dim:(head + 1) * head_dim])
             scores = (k[:, head // group, :] @ query) * scale
+            if head_scales is not None:
+                scores = scores * head_scales[head]
+            if sigmoid:
+                weights = torch.sigmoid(scores + (score_bias[head] if score_bias is not None else 0.0))
+                out[token, head * value_dim:(head + 1) * value_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
+                continue
             if slopes is not None:
                 scores = scores - slopes[head] * (position - keys).float()
             if log_bias is not None:
@@ -258,7 +311,8 @@ def head_norm_gate(raw, gate, weight, num_heads, eps, activation, out):
 
 def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, state, cu_seqlens, slot_ids, out,
                       max_query_len=0, head_decay=None, key_scale=1.0, positions=None, inv_freq=None, rotary_dim=0,
-                      removal_col=-1, decay_logits=None, decay_bias=None, decay_floor=0.0, key_eps=0.0, chunks=None):
+                      removal_col=-1, decay_logits=None, decay_bias=None, decay_floor=0.0, key_eps=0.0, chunks=None,
+                      gate_power=0.0, query_scale=1.0):
     """``state`` [slots, H, value dim, key dim] holds the transposed state of every head."""
     H, K, V = num_heads, key_dim, value_dim
     T = u.shape[0]
@@ -266,6 +320,7 @@ def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, 
     k = _f(u[:, k_col:k_col + H * K]).reshape(T, H, K).clone()
     v = _f(u[:, v_col:v_col + H * V]).reshape(T, H, V)
     delta = removal_col >= 0
+    gated = not delta and gate_power > 0
     if inv_freq is not None and rotary_dim > 0:
         half = rotary_dim // 2
         angle = positions.to(torch.float32)[:, None] * inv_freq[None, :]
@@ -275,6 +330,9 @@ def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, 
             a, b = x[..., :half], x[..., half:rotary_dim]
             return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., rotary_dim:]], dim=-1)
         q, k = rotate(q), rotate(k)
+    q = q * query_scale
+    if gated:
+        decay = torch.exp(F.logsigmoid(decay_logits + decay_bias) * gate_power).reshape(T, H, K)
     if delta:
         unit = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + key_eps)
         removal = torch.sigmoid(_f(u[:, removal_col:removal_col + H * K])).reshape(T, H, K)
@@ -289,6 +347,8 @@ def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, 
                 along = torch.einsum("hk,hkv->hv", unit[t], S)
                 S = decay[t][:, :, None] * S - (removal[t] * unit[t])[:, :, None] * along[:, None, :] \
                     + k[t][:, :, None] * v[t][:, None, :]
+            elif gated:
+                S = decay[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
             else:
                 S = head_decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
             out[t] = torch.einsum("hkv,hk->hv", S, q[t]).reshape(H * V)
@@ -327,8 +387,16 @@ def stream_add(h, rows, factor, vector):
         h += vector
 
 
-def add_layernorm(h, branches, vector, weight, bias, eps, out, rows=None):
+def add_layernorm(h, branches, vector, weight, bias, eps, out, rows=None, branch_norm=None):
     total = h.clone()
+    if branch_norm is not None:
+        summed = torch.zeros_like(h)
+        for tensor, factor in branches:
+            summed = summed + float(factor) * _f(tensor)
+        centred = summed - summed.mean(dim=-1, keepdim=True)
+        variance = (centred * centred).mean(dim=-1, keepdim=True)
+        total = total + centred / torch.sqrt(variance + branch_norm[2]) * branch_norm[0] + branch_norm[1]
+        branches = []
     for tensor, factor in branches:
         total = total + float(factor) * _f(tensor)
     if vector is not None:
@@ -475,7 +543,8 @@ NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supporte
          "conv1d_silu", "conv_state_update", "conv_step", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed",
          "add_scaled_rmsnorm", "polynorm", "tanh_rows", "head_norm_gate", "linear_state_scan",
          "embed_bigram", "stream_add", "add_layernorm", "clamped_glu", "latent_prepare", "head_linear", "rotate_heads",
-         "latent_attention_supported", "moe_route", "moe_plan", "moe_expert_gemm", "moe_combine"]
+         "latent_attention_supported", "moe_route", "moe_plan", "moe_expert_gemm", "moe_combine", "cast_rows",
+         "attention_prepare"]
 
 
 def install(monkeypatch):
