@@ -115,6 +115,125 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
   return 0;
 }
 
+// ---------------------------------------------------------------- a token's row made ready for attention
+// One workgroup a token; the row [q heads | k heads | v heads] is laid in LDS as float32 and everything below is
+// float32 arithmetic on that copy:
+//   * q_norm / k_norm (optional): the whole q projection (Hq * dh numbers), and the whole k projection, is divided by
+//     its root mean square (eps inside the root) and multiplied by a weight of that length, before rotation;
+//   * q and k are turned by the token's position (half-split pairs over the first rotary_dim dims, angle =
+//     (float)position * inv_freq[j]); q is written back in place, k goes to the token's cache cell;
+//   * the values are the v heads of the row or, with values_from_keys, the k heads as they were projected (before
+//     norm and rotation; dv = dh); with value_inv_freq they are turned by the position over all dv dims (half-split
+//     pairs, angle = (float)position * value_inv_freq[m]); they go to the token's transposed cache cell.
+template <typename T>
+__global__ void __launch_bounds__(256)
+attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, int dv, int values_from_keys,
+                         const int* __restrict__ positions, const float* __restrict__ inv_freq, int rotary_dim,
+                         const float* __restrict__ q_norm, const float* __restrict__ k_norm, float norm_eps,
+                         const float* __restrict__ value_inv_freq, const int* __restrict__ slot_mapping,
+                         T* __restrict__ k_base, T* __restrict__ v_base, long page_stride, int page_size) {
+  extern __shared__ float prepared_row[];
+  __shared__ float scratch[16];
+  const long token = blockIdx.x;
+  T* row = qkv + token * ld;
+  const float position = (float)positions[token];
+  const int q_cols = Hq * dh, k_cols = Hkv * dh;
+  const int v_cols = Hkv * dv;
+  float* q_lds = prepared_row;
+  float* k_lds = q_lds + q_cols;
+  float* v_lds = k_lds + k_cols;
+  float q_squares = 0.f, k_squares = 0.f;
+  for (int i = threadIdx.x; i < q_cols + k_cols; i += blockDim.x) {
+    const float x = to_float(row[i]);
+    prepared_row[i] = x;
+    if (i < q_cols) q_squares = fmaf(x, x, q_squares);
+    else k_squares = fmaf(x, x, k_squares);
+  }
+  for (int i = threadIdx.x; i < v_cols; i += blockDim.x)
+    v_lds[i] = to_float(values_from_keys ? row[q_cols + i] : row[q_cols + k_cols + i]);
+  if (q_norm) {
+    const float q_rms = sqrtf(block_sum(q_squares, scratch) / (float)q_cols + norm_eps);
+    const float k_rms = sqrtf(block_sum(k_squares, scratch) / (float)k_cols + norm_eps);
+    for (int i = threadIdx.x; i < q_cols; i += blockDim.x) q_lds[i] = q_lds[i] / q_rms * q_norm[i];
+    for (int i = threadIdx.x; i < k_cols; i += blockDim.x) k_lds[i] = k_lds[i] / k_rms * k_norm[i];
+  }
+  __syncthreads();
+  long cell = -1, page = 0;
+  int offset = 0;
+  if (slot_mapping) {
+    cell = slot_mapping[token];
+    page = cell / page_size;
+    offset = (int)(cell - page * page_size);
+  }
+  // q heads then k heads: a thread an element; the partner of a turned element is read from LDS, which nobody writes
+  const int half = rotary_dim / 2;
+  for (int item = threadIdx.x; item < q_cols + k_cols; item += blockDim.x) {
+    const int head = item / dh;
+    const int j = item - head * dh;
+    const float* x = prepared_row + (long)head * dh;
+    float value = x[j];
+    if (inv_freq && j < rotary_dim) {
+      const bool low = j < half;
+      const float angle = position * inv_freq[low ? j : j - half];
+      float sine, cosine;
+      sincosf(angle, &sine, &cosine);
+      const float partner = x[low ? j + half : j - half];
+      value = low ? value * cosine - partner * sine : value * cosine + partner * sine;
+    }
+    if (head < Hq) row[item] = from_float<T>(value);
+    else if (cell >= 0)
+      k_base[page * page_stride + ((long)(head - Hq) * page_size + offset) * dh + j] = from_float<T>(value);
+  }
+  if (cell >= 0) {
+    const int value_half = dv / 2;
+    for (int item = threadIdx.x; item < v_cols; item += blockDim.x) {
+      const int kvh = item / dv;
+      const int i = item - kvh * dv;
+      float value = v_lds[item];
+      if (value_inv_freq) {
+        const bool low = i < value_half;
+        const float angle = position * value_inv_freq[low ? i : i - value_half];
+        float sine, cosine;
+        sincosf(angle, &sine, &cosine);
+        const float partner = v_lds[kvh * dv + (low ? i + value_half : i - value_half)];
+        value = low ? value * cosine - partner * sine : value * cosine + partner * sine;
+      }
+      v_base[page * page_stride + ((long)kvh * dv + i) * page_size + offset] = from_float<T>(value);
+    }
+  }
+}
+
+extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq, int Hkv, int dh, int dv,
+                                    int values_from_keys, const int* positions, const float* inv_freq, int rotary_dim,
+                                    const float* q_norm, const float* k_norm, float norm_eps,
+                                    const float* value_inv_freq, const int* slot_mapping, void* k_base, void* v_base,
+                                    long page_stride, int page_size, hipStream_t stream) {
+  if (!qkv || !positions || T <= 0 || Hq <= 0 || Hkv <= 0 || dh <= 0 || dv <= 0) return ERR_BAD_ARGUMENT;
+  if (rotary_dim < 0 || rotary_dim > dh || (rotary_dim & 1) || (rotary_dim > 0 && !inv_freq)) return ERR_BAD_ARGUMENT;
+  if (values_from_keys && dv != dh) return ERR_BAD_ARGUMENT;
+  if (value_inv_freq && (dv & 1)) return ERR_BAD_ARGUMENT;
+  if ((q_norm == nullptr) != (k_norm == nullptr)) return ERR_BAD_ARGUMENT;
+  if (ld < (long)(Hq + Hkv) * dh + (values_from_keys ? 0L : (long)Hkv * dv)) return ERR_BAD_ARGUMENT;
+  if (slot_mapping && (!k_base || !v_base || page_size <= 0)) return ERR_BAD_ARGUMENT;
+  if (!inv_freq) rotary_dim = 0;
+  const size_t lds = ((size_t)(Hq + Hkv) * dh + (size_t)Hkv * dv) * sizeof(float);
+  if (lds > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  if (dtype == DT_F32)
+    attention_prepare_kernel<float><<<T, 256, lds, stream>>>((float*)qkv, ld, Hq, Hkv, dh, dv, values_from_keys, positions,
+                                                             inv_freq, rotary_dim, q_norm, k_norm, norm_eps,
+                                                             value_inv_freq, slot_mapping, (float*)k_base, (float*)v_base,
+                                                             page_stride, page_size);
+  else if (dtype == DT_BF16)
+    attention_prepare_kernel<bf16_t><<<T, 256, lds, stream>>>((bf16_t*)qkv, ld, Hq, Hkv, dh, dv, values_from_keys,
+                                                              positions, inv_freq, rotary_dim, q_norm, k_norm, norm_eps,
+                                                              value_inv_freq, slot_mapping, (bf16_t*)k_base,
+                                                              (bf16_t*)v_base, page_stride, page_size);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 // ---------------------------------------------------------------- paged attention, any size
 // Works for any head_dim <= 256, any page size, any group size, float32 and bfloat16; the float32 path of
 // the whole model uses it for prompts and for decoding alike.
@@ -127,6 +246,10 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 //   s -= r1 * ln(1 + r2 * (query position - key position)).
 // `sinks` (optional, float32 per query head, read by the merge kernel): exp(sink) is one more term of the softmax's
 //   denominator; it has no key and no value.
+// `head_scales` (optional, float32 per query head): s *= head_scales[head] behind the scale.
+// `sigmoid` (with an optional `score_bias`, float32 per query head): a visible key weighs sigmoid(s + score_bias[head])
+//   on its own and nothing is normalized: the kernels keep the maximum 0 for every group of keys, so every weight of
+//   the merges below is exp(0) = 1 and the sums are plain sums in the order of the keys; the merge does not divide.
 // dv: the width of a value head; the partial results and the output have dv dims a head.
 // The keys are cut into runs of PA_RUN by their absolute position.  One workgroup per (token, query head,
 // run): each of its four waves takes 64 keys of the run (lane i scores key i with a full dot product over
@@ -147,7 +270,8 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
                        int page_size, const int* __restrict__ block_tables, int max_pages,
                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
                        int window, const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
-                       float* __restrict__ partial) {
+                       float* __restrict__ partial, const float* __restrict__ head_scales,
+                       const float* __restrict__ score_bias, int sigmoid) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
   __shared__ __align__(16) float q_shared[ATT_MAX_DH];
   __shared__ float p_shared[PA_WAVES][WAVE];
@@ -192,11 +316,17 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
       for (int i = 0; i < dh; ++i) dot = fmaf(q_shared[i], to_float(k_row[i]), dot);
     }
     score = dot * scale;
+    if (head_scales) score *= head_scales[head];
     if (slopes) score = fmaf(-slopes[head], (float)(query_position - key), score);
     if (log_bias) score = fmaf(-log_bias[2 * head], log1pf(log_bias[2 * head + 1] * (float)(query_position - key)), score);
+    if (score_bias) score += score_bias[head];
   }
-  const float maximum = wave_max(score);                    // -inf for a wave without visible keys
-  const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
+  const float maximum = sigmoid ? 0.f : wave_max(score);    // -inf for a wave without visible keys
+  float p = 0.f;
+  if (visible) {
+    if (sigmoid) p = 1.0f / (1.0f + (FAST_EXP ? __expf(-score) : expf(-score)));
+    else p = FAST_EXP ? __expf(score - maximum) : expf(score - maximum);
+  }
   p_shared[wave][lane] = p;
   row_shared[wave][lane] = row_offset;
   offset_shared[wave][lane] = offset;
@@ -303,7 +433,8 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
                             const int* __restrict__ query_tiles, int tile_tokens, const int* __restrict__ cu_seqlens,
                             const int* __restrict__ positions, float scale, int window,
                             const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
-                            float* __restrict__ partial) {
+                            float* __restrict__ partial, const float* __restrict__ head_scales,
+                            const float* __restrict__ score_bias, int sigmoid) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
   extern __shared__ __align__(16) float tile_lds[];
   const int k_ld = dh + PT_PAD;                      // a key's row in LDS
@@ -430,11 +561,17 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       float score = -INFINITY;
       if (visible) {
         score = dot[i] * scale;
+        if (head_scales) score *= head_scales[head];
         if (slopes) score = fmaf(-slopes[head], (float)(position - key), score);
         if (log_bias) score = fmaf(-log_bias[2 * head], log1pf(log_bias[2 * head + 1] * (float)(position - key)), score);
+        if (score_bias) score += score_bias[head];
       }
-      const float maximum = wave_max_dpp(score);
-      const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
+      const float maximum = sigmoid ? 0.f : wave_max_dpp(score);
+      float p = 0.f;
+      if (visible) {
+        if (sigmoid) p = 1.0f / (1.0f + (FAST_EXP ? __expf(-score) : expf(-score)));
+        else p = FAST_EXP ? __expf(score - maximum) : expf(score - maximum);
+      }
       p_rows[i * p_ld + lane] = p;
       group_max[i][g] = maximum;
     }
@@ -531,7 +668,8 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
 template <typename T, bool FAST_EXP>
 __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, int Hq, int dh, int runs,
                                              const int* __restrict__ positions, int window,
-                                             const float* __restrict__ sinks, T* __restrict__ out, long out_ld) {
+                                             const float* __restrict__ sinks, T* __restrict__ out, long out_ld,
+                                             int sigmoid) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int query_position = positions[token];
@@ -561,7 +699,7 @@ __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, 
       denominator = denominator * keep + (FAST_EXP ? __expf(sink - larger) : expf(sink - larger));
       sum *= keep;
     }
-    out[token * out_ld + (long)head * dh + dim] = from_float<T>(sum / denominator);
+    out[token * out_ld + (long)head * dh + dim] = from_float<T>(sigmoid ? sum : sum / denominator);
   }
 }
 
@@ -606,7 +744,9 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
                                   const float* log_bias, const float* sinks,
                                   int max_seq_len, float* partial, long partial_floats, void* out, long out_ld,
                                   const int* query_tiles, int num_tiles, int tile_tokens, const int* cu_seqlens,
+                                  const float* head_scales, const float* score_bias, int sigmoid,
                                   hipStream_t stream) {
+  if ((score_bias && !sigmoid) || (sigmoid && sinks)) return ERR_BAD_ARGUMENT;
   if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || dv <= 0 || page_size <= 0 || max_pages <= 0 ||
       max_seq_len <= 0 || !partial)
     return ERR_BAD_ARGUMENT;
@@ -639,17 +779,19 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
 #define TILE_LAUNCH(T_, FAST_, DIMS_)                                                                                 \
   paged_attention_tile_kernel<T_, FAST_, DIMS_><<<tile_grid, PA_RUN, tile_lds, stream>>>(                              \
       (const T_*)q, q_ld, Hq, Hkv, dh, dv, (const T_*)k_base, (const T_*)v_base, page_stride, page_size, block_tables, \
-      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, log_bias, runs, partial)
+      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, log_bias, runs, partial,       \
+      head_scales, score_bias, sigmoid)
     if (tiled && dims == 1) TILE_LAUNCH(float, false, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(float, false, 2);
     else if (tiled) TILE_LAUNCH(float, false, 4);
     else
       paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
           (const float*)q, q_ld, Hq, Hkv, dh, dv, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial);
+          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial,
+          head_scales, score_bias, sigmoid);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dv, runs, positions, window, sinks, (float*)out, out_ld);
+        partial, Hq, dv, runs, positions, window, sinks, (float*)out, out_ld, sigmoid);
   } else if (dtype == DT_BF16) {
     if (tiled && dims == 1) TILE_LAUNCH(bf16_t, true, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(bf16_t, true, 2);
@@ -657,10 +799,11 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
     else
       paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
           (const bf16_t*)q, q_ld, Hq, Hkv, dh, dv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial);
+          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial,
+          head_scales, score_bias, sigmoid);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dv, runs, positions, window, sinks, (bf16_t*)out, out_ld);
+        partial, Hq, dv, runs, positions, window, sinks, (bf16_t*)out, out_ld, sigmoid);
   } else {
     return ERR_BAD_ARGUMENT;
   }

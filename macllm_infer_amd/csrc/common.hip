@@ -275,8 +275,19 @@ __device__ __forceinline__ long swiglu_gate_at(int i, int I, int tile) {
   return tile == 0 ? i : (long)(i / tile) * 2 * tile + i % tile;
 }
 
+// the gate's activation: 0 SiLU, 1 the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+// the same through the hardware's exponential: tanh(y) = 1 - 2 / (1 + e^(2y)); for results rounded to bfloat16 at once
+__device__ __forceinline__ float gelu_tanh_bf16_f(float z) {
+  const float y = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return z * (1.0f - __frcp_rn(1.0f + __expf(2.0f * y)));
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__ out, int I, int tile, long total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__ out, int I, int tile, long total,
+                              int activation) {
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (index >= total) return;
   const long t = index / I;
@@ -284,13 +295,14 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__
   const long at = swiglu_gate_at(i, I, tile);
   const float gate = to_float(gu[t * ld + at]);
   const float up = to_float(gu[t * ld + at + (tile == 0 ? I : tile)]);
-  out[index] = from_float<T>(silu_f(gate) * up);
+  out[index] = from_float<T>((activation == 1 ? gelu_tanh_f(gate) : silu_f(gate)) * up);
 }
 
 // bfloat16, eight elements a thread (I, ld and the addresses multiples of 8 elements; tile 0 or 8)
 typedef __bf16 common_bf16x8 __attribute__((ext_vector_type(8)));
 __global__ void __launch_bounds__(256)
-swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ out, int I, int tile, long total) {
+swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ out, int I, int tile, long total,
+                  int activation) {
   const long index = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (index >= total) return;
   const long t = index / I;
@@ -300,22 +312,49 @@ swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ o
   const common_bf16x8 up = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + at + (tile == 0 ? I : 8));
   common_bf16x8 result;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) result[j] = (bf16_t)(silu_bf16_f((float)gate[j]) * (float)up[j]);
+  for (int j = 0; j < 8; ++j)
+    result[j] = (bf16_t)((activation == 1 ? gelu_tanh_bf16_f((float)gate[j]) : silu_bf16_f((float)gate[j])) * (float)up[j]);
   *reinterpret_cast<common_bf16x8*>(out + index) = result;
 }
 
-extern "C" int mi_swiglu(const void* gu, int dtype, long ld, void* out, int T, int I, int tile, hipStream_t stream) {
-  if (T <= 0 || I <= 0 || ld < 2L * I || tile < 0 || (tile > 0 && I % tile != 0)) return ERR_BAD_ARGUMENT;
+extern "C" int mi_swiglu(const void* gu, int dtype, long ld, void* out, int T, int I, int tile, int activation,
+                         hipStream_t stream) {
+  if (T <= 0 || I <= 0 || ld < 2L * I || tile < 0 || (tile > 0 && I % tile != 0) || (activation != 0 && activation != 1))
+    return ERR_BAD_ARGUMENT;
   const long total = (long)T * I;
   const int blocks = (int)((total + 255) / 256);
   if (dtype == DT_BF16 && I % 8 == 0 && ld % 8 == 0 && (tile == 0 || tile == 8) && ((uintptr_t)gu % 16) == 0 &&
       ((uintptr_t)out % 16) == 0) {
     const int vec_blocks = (int)((total / 8 + 255) / 256);
-    swiglu_vec_kernel<<<vec_blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total);
+    swiglu_vec_kernel<<<vec_blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total, activation);
   } else if (dtype == DT_F32)
-    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, ld, (float*)out, I, tile, total);
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, ld, (float*)out, I, tile, total, activation);
   else if (dtype == DT_BF16)
-    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total);
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total, activation);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- float32 rows into a matrix of activations
+// out[t * ld + i] = (T)source[t * d + i]
+template <typename T>
+__global__ void cast_rows_kernel(const float* __restrict__ source, T* __restrict__ out, long ld, int d, long total) {
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= total) return;
+  const long t = index / d;
+  out[t * ld + (index - t * d)] = from_float<T>(source[index]);
+}
+
+extern "C" int mi_cast_rows(const float* source, void* out, int dtype, long ld, int T, int d, hipStream_t stream) {
+  if (!source || !out || T <= 0 || d <= 0 || ld < d) return ERR_BAD_ARGUMENT;
+  const long total = (long)T * d;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == DT_F32)
+    cast_rows_kernel<float><<<blocks, 256, 0, stream>>>(source, (float*)out, ld, d, total);
+  else if (dtype == DT_BF16)
+    cast_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>(source, (bf16_t*)out, ld, d, total);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();
@@ -610,23 +649,53 @@ __device__ __forceinline__ float branch_value(const NormBranch& branch, long at)
 template <typename TO>
 __global__ void __launch_bounds__(1024)
 add_layernorm_kernel(float* __restrict__ h, NormBranch b0, NormBranch b1, NormBranch b2, const float* __restrict__ vector,
-                     const float* __restrict__ weight, const float* __restrict__ bias, float eps, TO* __restrict__ out,
-                     const int* __restrict__ rows, int d) {
+                     const float* __restrict__ weight, const float* __restrict__ bias, float eps,
+                     const float* __restrict__ branch_weight, const float* __restrict__ branch_bias, float branch_eps,
+                     TO* __restrict__ out, const int* __restrict__ rows, int d) {
   extern __shared__ float wide_row[];
   __shared__ float scratch[16];
   const long out_row = blockIdx.x;
   const long row = rows ? (long)rows[out_row] : out_row;
   float sum = 0.f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    const long at = row * d + i;
-    float v = h[at];
-    v += branch_value(b0, at);
-    v += branch_value(b1, at);
-    v += branch_value(b2, at);
-    if (vector) v += vector[i];
-    if (!rows) h[at] = v;
-    wide_row[i] = v;
-    sum += v;
+  if (branch_weight) {
+    // the branches' sum goes through a layer norm of its own on its way into the stream: the sum is laid in LDS,
+    // its mean and the variance of its deviations are taken as below, and the normed row is added to h
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      const long at = row * d + i;
+      float v = branch_value(b0, at);
+      v += branch_value(b1, at);
+      v += branch_value(b2, at);
+      wide_row[i] = v;
+      sum += v;
+    }
+    const float branch_mean = block_sum(sum, scratch) / (float)d;
+    float branch_squares = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      const float centred = wide_row[i] - branch_mean;
+      branch_squares += centred * centred;
+    }
+    const float branch_denominator = sqrtf(block_sum(branch_squares, scratch) / (float)d + branch_eps);
+    sum = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      const long at = row * d + i;
+      float v = h[at] + ((wide_row[i] - branch_mean) / branch_denominator * branch_weight[i] + branch_bias[i]);
+      if (vector) v += vector[i];
+      h[at] = v;
+      wide_row[i] = v;
+      sum += v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      const long at = row * d + i;
+      float v = h[at];
+      v += branch_value(b0, at);
+      v += branch_value(b1, at);
+      v += branch_value(b2, at);
+      if (vector) v += vector[i];
+      if (!rows) h[at] = v;
+      wide_row[i] = v;
+      sum += v;
+    }
   }
   if (!out) return;
   const float mean = block_sum(sum, scratch) / (float)d;
@@ -644,17 +713,22 @@ add_layernorm_kernel(float* __restrict__ h, NormBranch b0, NormBranch b1, NormBr
 
 extern "C" int mi_add_layernorm(float* h, const void* rows0, int dtype0, float factor0, const void* rows1, int dtype1,
                                 float factor1, const void* rows2, int dtype2, float factor2, const float* vector,
-                                const float* weight, const float* bias, float eps, void* out, int out_dtype,
+                                const float* weight, const float* bias, float eps, const float* branch_weight,
+                                const float* branch_bias, float branch_eps, void* out, int out_dtype,
                                 const int* rows, int n_rows, int d, hipStream_t stream) {
-  if (!h || !weight || !bias || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  if (!h || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  if (out && (!weight || !bias)) return ERR_BAD_ARGUMENT;
+  if (branch_weight && (!branch_bias || rows || !rows0)) return ERR_BAD_ARGUMENT;
   if ((size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   const NormBranch b0 = {rows0, dtype0, factor0}, b1 = {rows1, dtype1, factor1}, b2 = {rows2, dtype2, factor2};
   const int threads = (d > 2048 && n_rows <= 512) ? 1024 : 256;
   const size_t lds = (size_t)d * sizeof(float);
   if (out_dtype == DT_F32)
-    add_layernorm_kernel<float><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, (float*)out, rows, d);
+    add_layernorm_kernel<float><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, branch_weight,
+                                                                  branch_bias, branch_eps, (float*)out, rows, d);
   else if (out_dtype == DT_BF16)
-    add_layernorm_kernel<bf16_t><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, (bf16_t*)out, rows, d);
+    add_layernorm_kernel<bf16_t><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, branch_weight,
+                                                                   branch_bias, branch_eps, (bf16_t*)out, rows, d);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();

@@ -3,13 +3,16 @@
 //
 //   retention        S <- decay[h] * S + k v^T                         o = S^T q
 //   delta rule       S <- diag(w) S - (a * u)(u^T S) + k v^T           o = S^T r      (both products on the old S)
+//   gated decay      S <- diag(w) S + k v^T                            o = S^T q      (w a gate of the token)
 //
 // with S [dk, dv] per head in float32, carried from token to token in the request's state slot.  What enters the
 // recurrence is formed in float32 from the projection's rows inside the scan:
 //   retention : q and k turned by position (half-split rotation of the first rotary_dim dims, angle =
 //               (float)position * inv_freq[j]), then k * key_scale;
 //   delta rule: u = k / sqrt(sum k^2 + key_eps), a = sigmoid(removal columns),
-//               w = exp(-decay_floor * sigmoid(decay_logits + decay_bias)).
+//               w = exp(-decay_floor * sigmoid(decay_logits + decay_bias));
+//   gated decay: w = sigmoid(decay_logits + decay_bias)^gate_power = exp(gate_power * log sigmoid(.)) per head and
+//               key channel, q * query_scale.
 //
 // The state is stored transposed, [slot][head][dv][dk]: a column of S (all key channels of one value channel)
 // evolves on its own,
@@ -25,7 +28,9 @@
 // lane) that the step carries), so that the tokens of one prompt are worked on side by side:
 //   local   every chunk but a lane's last, from an empty state: the state B the chunk's own tokens leave, and for
 //           the delta rule the chunk's transition P = A_last ... A_first (A_t = diag(w_t) - (a_t u_t) u_t^T), whose
-//           column i is what the same recurrence without keys makes of the unit vector e_i: dk more columns;
+//           column i is what the same recurrence without keys makes of the unit vector e_i: dk more columns; for
+//           the gated decay the transition is diagonal, the product of the chunk's w, which is what the recurrence
+//           without keys makes of the vector of ones: one more column;
 //   carry   per lane, chunk after chunk: S_start(c + 1) = P_c S_start(c) + B_c (retention: P_c = decay^tokens),
 //           beginning with the request's state; every chunk's starting state is kept;
 //   scan    every chunk from its starting state: the outputs, and behind a lane's last chunk the state of the request.
@@ -58,6 +63,7 @@ struct ScanArgs {
   long logits_ld;
   const float* decay_bias;          // [H * dk]
   float decay_floor, key_eps;
+  float gate_power, query_scale;    // gated decay: the gate's exponent; what q is multiplied by (every kind)
   int R, per_lane, columns, stage;  // lanes a column, key channels a lane, columns a workgroup, tokens a stage
   const int* chunks;                // passes over chunks: [chunks, 4] = (lane, first row, tokens, index in the lane)
   const int* lane_chunks;           // [lanes, 2] = (first chunk, chunks)
@@ -65,11 +71,17 @@ struct ScanArgs {
   float* start;                     // [chunks, H, dv, dk]: every chunk's starting state
 };
 
+#define LS_RETENTION 0              // the kinds of recurrence
+#define LS_DELTA 1
+#define LS_GATED 2
+
 #define LS_WHOLE 0                  // a lane from and into its request's state
 #define LS_LOCAL 1                  // a chunk from an empty state (and the unit vectors): no outputs
 #define LS_CHUNK 2                  // a chunk from its starting state
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+// log(sigmoid(x)) = min(x, 0) - log1p(exp(-|x|)): finite for any finite x
+__device__ __forceinline__ float log_sigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
 // sum over the R neighbouring lanes of a column (R a power of two up to 64).  A constant R up to 16 stays inside a
 // row of 16 lanes, where the data-parallel primitives exchange lanes without a trip through the LDS crossbar:
@@ -100,9 +112,11 @@ __device__ __forceinline__ float dot4(const float4 a, const float* s) {
 // R_CONST: the lanes of a column when the launch knows them at compile time (1 .. 16), 0: a.R.
 // PL: key channels a lane; a lane keeps 16 / PL neighbouring columns (their states in 16 registers), so that the
 // token's vectors come out of LDS once for all of them.  PL = 16: one column, a.per_lane (<= 16) channels of it.
-template <typename T, bool DELTA, int MODE, int R_CONST, int PL>
+template <typename T, int KIND, int MODE, int R_CONST, int PL>
 __global__ void __launch_bounds__(MODE == LS_WHOLE ? LS_THREADS : LS_PASS_THREADS)
 linear_state_scan_kernel(const ScanArgs a) {
+  constexpr bool DELTA = KIND == LS_DELTA;
+  constexpr bool GATED = KIND == LS_GATED;
   constexpr int CPL = LS_MAX_PER_LANE / PL;              // columns a lane
   extern __shared__ __align__(16) float stage_lds[];
   const int head = blockIdx.y;
@@ -130,14 +144,15 @@ linear_state_scan_kernel(const ScanArgs a) {
   const int per_lane = PL < LS_MAX_PER_LANE ? PL : a.per_lane;   // a multiple of 4
   const int dk = a.dk, dv = a.dv;
   const int padded = R * per_lane;                       // a vector's length in LDS; channels past dk hold zeros
-  const int vectors = DELTA ? 5 : 2;
+  const int vectors = DELTA ? 5 : GATED ? 3 : 2;
   const int token_floats = vectors * padded + ((a.columns + 3) & ~3);
   const int group = tid / R;                             // the lanes of one run of CPL columns
   const int sub = tid - group * R;
   const int column_in_group = group * CPL;               // the first of this lane's columns among the workgroup's
   const int column0 = blockIdx.z * a.columns + column_in_group;
-  // the local pass of the delta rule carries dk more columns: the transition's, which start as the unit vectors
-  const int total_columns = (MODE == LS_LOCAL && DELTA) ? dv + dk : dv;
+  // the local pass of the delta rule carries dk more columns: the transition's, which start as the unit vectors;
+  // that of the gated decay one more: the diagonal transition, which starts as ones
+  const int total_columns = MODE == LS_LOCAL ? (DELTA ? dv + dk : GATED ? dv + 1 : dv) : dv;
   const bool in_group = column_in_group < a.columns;
   const int channel0 = sub * per_lane;
   const T* rows = (const T*)a.u;
@@ -155,11 +170,11 @@ linear_state_scan_kernel(const ScanArgs a) {
     for (int e = 0; e < PL; ++e) {
       const int channel = channel0 + e;
       const bool held = mine && e < per_lane && channel < dk;
-      if (MODE == LS_LOCAL) s[c][e] = (held && channel == column - dv) ? 1.f : 0.f;
+      if (MODE == LS_LOCAL) s[c][e] = (held && (GATED ? column == dv : channel == column - dv)) ? 1.f : 0.f;
       else s[c][e] = held ? from[channel] : 0.f;
     }
   }
-  const float decay = DELTA ? 0.f : a.head_decay[head];
+  const float decay = KIND == LS_RETENTION ? a.head_decay[head] : 0.f;
   const int half = a.rotary_dim / 2;
 
   for (int stage_first = first_token; stage_first < end_token; stage_first += a.stage) {
@@ -195,10 +210,15 @@ linear_state_scan_kernel(const ScanArgs a) {
             kx = low ? kx * cosine - k_pair * sine : kx * cosine + k_pair * sine;
           }
           kx *= a.key_scale;
+          if (GATED)
+            w = expf(a.gate_power * log_sigmoid_f(a.decay_logits[token * a.logits_ld + head * dk + channel] +
+                                                  a.decay_bias[head * dk + channel]));
         }
+        qx *= a.query_scale;
       }
       q_lds[channel] = qx;
       q_lds[padded + channel] = kx;
+      if (GATED) q_lds[2 * padded + channel] = w;
       if (DELTA) {
         q_lds[2 * padded + channel] = w;
         q_lds[4 * padded + channel] = removal;             // times the unit key below
@@ -273,6 +293,21 @@ linear_state_scan_kernel(const ScanArgs a) {
                 s[c][4 * g + 3] = fmaf(k4.w, value[c], fmaf(-au4.w, along[c], w4.w * s[c][4 * g + 3]));
               }
             }
+        } else if (GATED) {
+          const float* w_lds = k_lds + padded;
+#pragma unroll
+          for (int g = 0; g < PL / 4; ++g)
+            if (4 * g < per_lane) {
+              const float4 k4 = *reinterpret_cast<const float4*>(k_lds + 4 * g);
+              const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 4 * g);
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) {
+                s[c][4 * g + 0] = fmaf(k4.x, value[c], w4.x * s[c][4 * g + 0]);
+                s[c][4 * g + 1] = fmaf(k4.y, value[c], w4.y * s[c][4 * g + 1]);
+                s[c][4 * g + 2] = fmaf(k4.z, value[c], w4.z * s[c][4 * g + 2]);
+                s[c][4 * g + 3] = fmaf(k4.w, value[c], w4.w * s[c][4 * g + 3]);
+              }
+            }
         } else {
 #pragma unroll
           for (int g = 0; g < PL / 4; ++g)
@@ -332,9 +367,11 @@ linear_state_scan_kernel(const ScanArgs a) {
 // (P's column i is row dv + i of what the local pass left); every chunk's starting state goes to ``start``.
 #define LS_CARRY_COLUMNS 4
 
-template <bool DELTA>
+template <int KIND>
 __global__ void __launch_bounds__(LS_THREADS)
 linear_state_carry_kernel(const ScanArgs a) {
+  constexpr bool DELTA = KIND == LS_DELTA;
+  constexpr bool GATED = KIND == LS_GATED;
   extern __shared__ __align__(16) float carry_lds[];       // [LS_CARRY_COLUMNS][dk]
   const int lane_of_step = blockIdx.x;
   const int head = blockIdx.y;
@@ -343,7 +380,7 @@ linear_state_carry_kernel(const ScanArgs a) {
   if (count <= 0) return;
   const int dk = a.dk, dv = a.dv;
   const int column0 = blockIdx.z * LS_CARRY_COLUMNS;
-  const int total_columns = DELTA ? dv + dk : dv;
+  const int total_columns = DELTA ? dv + dk : GATED ? dv + 1 : dv;
   const float* state = a.state + ((long)a.slot_ids[lane_of_step] * a.H + head) * dv * dk;
   for (int index = threadIdx.x; index < LS_CARRY_COLUMNS * dk; index += blockDim.x) {
     const int c = index / dk, m = index - c * dk;
@@ -352,11 +389,11 @@ linear_state_carry_kernel(const ScanArgs a) {
     if (column0 + c < dv) a.start[(((long)first_chunk * a.H + head) * dv + column0 + c) * dk + m] = value;
   }
   __syncthreads();
-  const float decay = DELTA ? 0.f : a.head_decay[head];
+  const float decay = KIND == LS_RETENTION ? a.head_decay[head] : 0.f;
   for (int chunk = first_chunk; chunk < first_chunk + count - 1; ++chunk) {
     const float* local = a.local + ((long)chunk * a.H + head) * total_columns * dk;
     float* start = a.start + ((long)(chunk + 1) * a.H + head) * dv * dk;
-    const float shrink = DELTA ? 0.f : powf(decay, (float)a.chunks[4 * chunk + 2]);
+    const float shrink = KIND == LS_RETENTION ? powf(decay, (float)a.chunks[4 * chunk + 2]) : 0.f;
     // more key channels than threads: rounds of blockDim.x channels (the new values wait in registers of the round)
     for (int m0 = 0; m0 < dk; m0 += blockDim.x) {
       const int m = m0 + threadIdx.x;
@@ -380,8 +417,10 @@ linear_state_carry_kernel(const ScanArgs a) {
             }
           }
         } else {
+          // retention: one number a chunk; gated decay: channel m's product of the chunk's gates
+          const float through = GATED ? local[(long)dv * dk + m] : shrink;
 #pragma unroll
-          for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = shrink * carry_lds[c * dk + m];
+          for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = through * carry_lds[c * dk + m];
         }
 #pragma unroll
         for (int c = 0; c < LS_CARRY_COLUMNS; ++c)
@@ -414,12 +453,13 @@ static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, 
                      int dv, float* state, const int* cu_seqlens, const int* slot_ids, int lanes, float* out, long out_ld,
                      const float* head_decay, float key_scale, const int* positions, const float* inv_freq,
                      int rotary_dim, const float* decay_logits, long logits_ld, const float* decay_bias,
-                     float decay_floor, float key_eps) {
+                     float decay_floor, float key_eps, float gate_power, float query_scale) {
   if (!u || !state || !cu_seqlens || !slot_ids || !out || lanes <= 0 || H <= 0 || dk <= 0 || dv <= 0)
     return ERR_BAD_ARGUMENT;
   const bool delta = removal_col >= 0;
-  if (delta && (!decay_logits || !decay_bias || logits_ld < (long)H * dk)) return ERR_BAD_ARGUMENT;
-  if (!delta && !head_decay) return ERR_BAD_ARGUMENT;
+  const bool gated = !delta && gate_power > 0.f;
+  if ((delta || gated) && (!decay_logits || !decay_bias || logits_ld < (long)H * dk)) return ERR_BAD_ARGUMENT;
+  if (!delta && !gated && !head_decay) return ERR_BAD_ARGUMENT;
   if (inv_freq && (!positions || rotary_dim <= 0 || rotary_dim > dk || (rotary_dim & 1))) return ERR_BAD_ARGUMENT;
   if (out_ld < (long)H * dv) return ERR_BAD_ARGUMENT;
   if (dk > LS_MAX_PER_LANE * WAVE || H > 65535 || lanes > 0x7fffffff) return ERR_UNSUPPORTED_SIZE;
@@ -428,6 +468,7 @@ static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, 
   a.out = out; a.out_ld = out_ld; a.head_decay = head_decay; a.key_scale = key_scale; a.positions = positions;
   a.inv_freq = inv_freq; a.rotary_dim = inv_freq ? rotary_dim : 0; a.decay_logits = decay_logits;
   a.logits_ld = logits_ld; a.decay_bias = decay_bias; a.decay_floor = decay_floor; a.key_eps = key_eps;
+  a.gate_power = gate_power; a.query_scale = query_scale;
   a.chunks = nullptr; a.lane_chunks = nullptr; a.local = nullptr; a.start = nullptr;
   int R = 1;
   while (R * LS_MAX_PER_LANE < dk) R *= 2;
@@ -437,12 +478,12 @@ static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, 
 }
 
 // columns a workgroup of ``threads`` threads takes of ``total_columns``, the tokens of a stage and its bytes in LDS
-static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, int longest, size_t* lds, int* splits) {
+static int scan_shape(ScanArgs& a, int threads, int total_columns, int kind, int longest, size_t* lds, int* splits) {
   a.columns = threads / a.R;
   if (a.columns > total_columns) a.columns = total_columns;
   *splits = (total_columns + a.columns - 1) / a.columns;
   if (*splits > 65535) return ERR_UNSUPPORTED_SIZE;
-  const int token_floats = (delta ? 5 : 2) * a.R * a.per_lane + ((a.columns + 3) & ~3);
+  const int token_floats = (kind == LS_DELTA ? 5 : kind == LS_GATED ? 3 : 2) * a.R * a.per_lane + ((a.columns + 3) & ~3);
   int stage = LS_STAGE_BYTES / (token_floats * (int)sizeof(float));
   if (stage > LS_STAGE_MOST) stage = LS_STAGE_MOST;
   if (longest > 0 && stage > longest) stage = longest;
@@ -455,11 +496,13 @@ static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, i
 #define LS_LAUNCH_R(MODE_, R_, PL_, grid_, threads_, lds_)                                                         \
   do {                                                                                                            \
     if (dtype == DT_F32) {                                                                                        \
-      if (delta) linear_state_scan_kernel<float, true, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);     \
-      else linear_state_scan_kernel<float, false, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);          \
+      if (kind == LS_DELTA) linear_state_scan_kernel<float, LS_DELTA, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a); \
+      else if (kind == LS_GATED) linear_state_scan_kernel<float, LS_GATED, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a); \
+      else linear_state_scan_kernel<float, LS_RETENTION, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);   \
     } else {                                                                                                      \
-      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);    \
-      else linear_state_scan_kernel<bf16_t, false, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);         \
+      if (kind == LS_DELTA) linear_state_scan_kernel<bf16_t, LS_DELTA, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a); \
+      else if (kind == LS_GATED) linear_state_scan_kernel<bf16_t, LS_GATED, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a); \
+      else linear_state_scan_kernel<bf16_t, LS_RETENTION, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);  \
     }                                                                                                             \
   } while (0)
 // the walk from end to end: one column a lane, up to 16 channels of it
@@ -491,18 +534,19 @@ extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col
                                     int lanes, float* out, long out_ld, int max_query_len, const float* head_decay,
                                     float key_scale, const int* positions, const float* inv_freq, int rotary_dim,
                                     const float* decay_logits, long logits_ld, const float* decay_bias,
-                                    float decay_floor, float key_eps, hipStream_t stream) {
+                                    float decay_floor, float key_eps, float gate_power, float query_scale,
+                                    hipStream_t stream) {
   if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_ARGUMENT;
   ScanArgs a;
   int code = scan_args(a, u, ld, q_col, k_col, v_col, removal_col, H, dk, dv, state, cu_seqlens, slot_ids, lanes, out,
                        out_ld, head_decay, key_scale, positions, inv_freq, rotary_dim, decay_logits, logits_ld,
-                       decay_bias, decay_floor, key_eps);
+                       decay_bias, decay_floor, key_eps, gate_power, query_scale);
   if (code) return code;
-  const bool delta = removal_col >= 0;
+  const int kind = removal_col >= 0 ? LS_DELTA : gate_power > 0.f ? LS_GATED : LS_RETENTION;
   const int threads = max_query_len == 1 ? WAVE : LS_THREADS;
   size_t lds;
   int splits;
-  code = scan_shape(a, threads, dv, delta, max_query_len, &lds, &splits);
+  code = scan_shape(a, threads, dv, kind, max_query_len, &lds, &splits);
   if (code) return code;
   const dim3 grid(lanes, H, splits);
   LS_LAUNCH_WHOLE(grid, threads, lds);
@@ -511,8 +555,8 @@ extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col
 }
 
 // floats of the two workspaces of the passes over ``chunks`` chunks
-extern "C" long mi_linear_state_local_floats(int chunks, int H, int dk, int dv, int delta) {
-  return (long)chunks * H * (delta ? dv + dk : dv) * dk;
+extern "C" long mi_linear_state_local_floats(int chunks, int H, int dk, int dv, int kind) {
+  return (long)chunks * H * (kind == LS_DELTA ? dv + dk : kind == LS_GATED ? dv + 1 : dv) * dk;
 }
 extern "C" long mi_linear_state_start_floats(int chunks, int H, int dk, int dv) { return (long)chunks * H * dv * dk; }
 
@@ -524,17 +568,18 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
                                             long out_ld, int chunk_tokens, const float* head_decay, float key_scale,
                                             const int* positions, const float* inv_freq, int rotary_dim,
                                             const float* decay_logits, long logits_ld, const float* decay_bias,
-                                            float decay_floor, float key_eps, const int* chunks, const int* lane_chunks,
+                                            float decay_floor, float key_eps, float gate_power, float query_scale,
+                                            const int* chunks, const int* lane_chunks,
                                             int num_chunks, float* local, float* start, hipStream_t stream) {
   if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_ARGUMENT;
   if (!chunks || !lane_chunks || num_chunks <= 0 || !local || !start || chunk_tokens <= 0) return ERR_BAD_ARGUMENT;
   ScanArgs a;
   int code = scan_args(a, u, ld, q_col, k_col, v_col, removal_col, H, dk, dv, state, cu_seqlens, slot_ids, lanes, out,
                        out_ld, head_decay, key_scale, positions, inv_freq, rotary_dim, decay_logits, logits_ld,
-                       decay_bias, decay_floor, key_eps);
+                       decay_bias, decay_floor, key_eps, gate_power, query_scale);
   if (code) return code;
   a.chunks = chunks; a.lane_chunks = lane_chunks; a.local = local; a.start = start;
-  const bool delta = removal_col >= 0;
+  const int kind = removal_col >= 0 ? LS_DELTA : gate_power > 0.f ? LS_GATED : LS_RETENTION;
   size_t lds;
   int splits;
   // the passes spread a column over more lanes than the walk from end to end: up to LS_PASS_LANES, four key
@@ -551,7 +596,8 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
     columns_a_lane = LS_MAX_PER_LANE / channels;
   }
   // local: the chunks' own states (and transitions)
-  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, kind == LS_DELTA ? dv + dk : kind == LS_GATED ? dv + 1 : dv, kind,
+                    chunk_tokens, &lds, &splits);
   if (code) return code;
   // no more waves than the columns fill
   int threads = (((a.columns + columns_a_lane - 1) / columns_a_lane * a.R + WAVE - 1) / WAVE) * WAVE;
@@ -564,11 +610,12 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
   int carry_threads = ((dk + WAVE - 1) / WAVE) * WAVE;
   if (carry_threads > LS_THREADS) carry_threads = LS_THREADS;
   const size_t carry_lds = (size_t)LS_CARRY_COLUMNS * dk * sizeof(float);
-  if (delta) linear_state_carry_kernel<true><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
-  else linear_state_carry_kernel<false><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
+  if (kind == LS_DELTA) linear_state_carry_kernel<LS_DELTA><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
+  else if (kind == LS_GATED) linear_state_carry_kernel<LS_GATED><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
+  else linear_state_carry_kernel<LS_RETENTION><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
   RETURN_IF_LAUNCH_FAILED();
   // scan: the outputs, and the requests' states behind their last chunks
-  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, dv, kind, chunk_tokens, &lds, &splits);
   if (code) return code;
   threads = (((a.columns + columns_a_lane - 1) / columns_a_lane * a.R + WAVE - 1) / WAVE) * WAVE;
   if (threads < LS_THREADS) threads = LS_THREADS;
