@@ -158,3 +158,12 @@ def forward(tokens, tensors, raw, stream_after=None):
             stream_after.append(x)
     x = layer_norm(x, W["final.norm"], W["final.norm.b"], eps)
     return x @ W["head"].T * raw.get("logit_scale", 1.0)
+
+
+def greedy(tokens, tensors, raw, count):
+    """``count`` tokens, each the most likely one after everything before it."""
+    tokens, out = list(tokens), []
+    for _ in range(count):
+        out.append(int(forward(tokens, tensors, raw)[-1].argmax()))
+        tokens.append(out[-1])
+    return out
