@@ -3,11 +3,41 @@ It shares no code with the package and is what the tests compare the engine with
 
 Notation: x [T, d] rows of one sequence, positions 0 .. T - 1 (or ``positions``), W tensors by stored name.
 """
+import contextlib
 import math
 
 import torch
 
 F64 = torch.float64
+
+# Inside ``activations_rounded_to(torch.bfloat16)`` every activation that a 16-bit engine keeps in 16 bits between
+# two kernels (normed rows, projected rows, turned queries, keys and values, attended rows, gated rows, the
+# feed-forward's activations, each branch's output, the rows that enter the mix before a pass) is rounded to that
+# dtype and widened again; sums, weights of keys, norm statistics, decays, the recurrence and the residual stream
+# stay exact.  How far that moves the logits is what 16-bit activations cost on a given set of weights: the model's
+# conditioning, not a kernel's doing.  With ``dither`` (a torch.Generator) every value is first moved by a random
+# fraction of its last kept bit, so that several runs give several samples of the rounding noise.
+_ROUND_TO = None
+_DITHER = None
+
+
+@contextlib.contextmanager
+def activations_rounded_to(dtype, dither=None):
+    global _ROUND_TO, _DITHER
+    before = (_ROUND_TO, _DITHER)
+    _ROUND_TO, _DITHER = dtype, dither
+    try:
+        yield
+    finally:
+        _ROUND_TO, _DITHER = before
+
+
+def _r(x):
+    if _ROUND_TO is None:
+        return x
+    if _DITHER is not None:
+        x = x * (1.0 + (torch.rand(x.shape, generator=_DITHER).to(F64) - 0.5) * 2.0 ** -8)
+    return x.to(_ROUND_TO).to(F64)
 
 
 def layer_norm(x, weight, bias, eps):
@@ -54,12 +84,12 @@ def sigmoid_attention(h, prefix, W, mixer, positions=None):
     T = h.shape[0]
     positions = torch.arange(T) if positions is None else positions
     heads, groups, dim = mixer["heads"], mixer["kv_heads"], mixer["dim"]
-    q = (h @ W[f"{prefix}.q"].T + W[f"{prefix}.q.b"]).reshape(T, heads, dim)
-    k = (h @ W[f"{prefix}.k"].T + W[f"{prefix}.k.b"]).reshape(T, groups, dim)
+    q = _r(h @ W[f"{prefix}.q"].T + W[f"{prefix}.q.b"]).reshape(T, heads, dim)
+    k = _r(h @ W[f"{prefix}.k"].T + W[f"{prefix}.k.b"]).reshape(T, groups, dim)
     v = k
     if mixer.get("rot") is not None:
         freq = frequencies(mixer["rot"]["base"], mixer["rot"]["dims"], mixer["rot"].get("scaling"))
-        q, k = turn(q, positions, freq, mixer["rot"]["dims"]), turn(k, positions, freq, mixer["rot"]["dims"])
+        q, k = _r(turn(q, positions, freq, mixer["rot"]["dims"])), _r(turn(k, positions, freq, mixer["rot"]["dims"]))
     seen = positions[None, :] <= positions[:, None]
     out = torch.zeros(T, heads, dim, dtype=F64)
     for head in range(heads):
@@ -67,7 +97,7 @@ def sigmoid_attention(h, prefix, W, mixer, positions=None):
         score = (q[:, head] @ k[:, group].T) * mixer["scale"] * W[f"{prefix}.temp"][head]
         weight = torch.sigmoid(score + W[f"{prefix}.pb"][head]) * seen
         out[:, head] = weight @ v[:, group]
-    return out.reshape(T, heads * dim) @ W[f"{prefix}.o"].T + W[f"{prefix}.o.b"]
+    return _r(_r(out).reshape(T, heads * dim) @ W[f"{prefix}.o"].T + W[f"{prefix}.o.b"])
 
 
 def softmax_attention(h, prefix, W, mixer, eps, positions=None):
@@ -76,31 +106,31 @@ def softmax_attention(h, prefix, W, mixer, eps, positions=None):
     positions = torch.arange(T) if positions is None else positions
     heads, groups, dim, vdim = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
     rot = mixer["rot"]
-    q = rms_norm(h @ W[f"{prefix}.q"].T, W[f"{prefix}.q.norm"], eps).reshape(T, heads, dim)
-    k = rms_norm(h @ W[f"{prefix}.k"].T, W[f"{prefix}.k.norm"], eps).reshape(T, groups, dim)
-    v = (h @ W[f"{prefix}.v"].T).reshape(T, groups, vdim)
+    q = rms_norm(_r(h @ W[f"{prefix}.q"].T), W[f"{prefix}.q.norm"], eps).reshape(T, heads, dim)
+    k = rms_norm(_r(h @ W[f"{prefix}.k"].T), W[f"{prefix}.k.norm"], eps).reshape(T, groups, dim)
+    v = _r(h @ W[f"{prefix}.v"].T).reshape(T, groups, vdim)
     freq = frequencies(rot["base"], rot["dims"], rot.get("scaling"))
-    q, k = turn(q, positions, freq, rot["dims"]), turn(k, positions, freq, rot["dims"])
+    q, k = _r(turn(q, positions, freq, rot["dims"])), _r(turn(k, positions, freq, rot["dims"]))
     value_freq = frequencies(rot["base"], vdim)
-    v = turn(v, positions, value_freq, vdim)
+    v = _r(turn(v, positions, value_freq, vdim))
     seen = positions[None, :] <= positions[:, None]
     out = torch.zeros(T, heads, vdim, dtype=F64)
     for head in range(heads):
         group = head // (heads // groups)
         score = ((q[:, head] @ k[:, group].T) * mixer["scale"]).masked_fill(~seen, -math.inf)
         out[:, head] = torch.softmax(score, dim=-1) @ v[:, group]
-    out = turn(out, positions, value_freq, vdim, backwards=True)
-    return out.reshape(T, heads * vdim) @ W[f"{prefix}.o"].T
+    out = _r(turn(_r(out), positions, value_freq, vdim, backwards=True))
+    return _r(out.reshape(T, heads * vdim) @ W[f"{prefix}.o"].T)
 
 
 def gated_linear(h, prefix, W, mixer, eps, state=None):
     """S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head; returns (rows, final state [H, dk, dv])."""
     T = h.shape[0]
     heads, dim, vdim = mixer["heads"], mixer["dim"], mixer["vdim"]
-    q = (h @ W[f"{prefix}.q"].T * dim ** -0.5).reshape(T, heads, dim)
-    k = (h @ W[f"{prefix}.k"].T).reshape(T, heads, dim)
-    v = (h @ W[f"{prefix}.v"].T).reshape(T, heads, vdim)
-    z = (h @ W[f"{prefix}.a1"].T) @ W[f"{prefix}.a2"].T + W[f"{prefix}.a2.b"]
+    q = (_r(h @ W[f"{prefix}.q"].T) * dim ** -0.5).reshape(T, heads, dim)
+    k = _r(h @ W[f"{prefix}.k"].T).reshape(T, heads, dim)
+    v = _r(h @ W[f"{prefix}.v"].T).reshape(T, heads, vdim)
+    z = _r(h @ W[f"{prefix}.a1"].T) @ W[f"{prefix}.a2"].T + W[f"{prefix}.a2.b"]
     alpha = (torch.sigmoid(z) ** (1.0 / mixer["tau"])).reshape(T, heads, dim)
     S = torch.zeros(heads, dim, vdim, dtype=F64) if state is None else state.clone()
     o = torch.zeros(T, heads, vdim, dtype=F64)
@@ -108,18 +138,18 @@ def gated_linear(h, prefix, W, mixer, eps, state=None):
         S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
         o[t] = torch.einsum("hkv,hk->hv", S, q[t])
     o = rms_norm(o, W[f"{prefix}.norm"], eps)
-    gate = h @ W[f"{prefix}.g"].T
-    return (o.reshape(T, heads * vdim) * (gate * torch.sigmoid(gate))) @ W[f"{prefix}.o"].T, S
+    gate = _r(h @ W[f"{prefix}.g"].T)
+    return _r(_r(o.reshape(T, heads * vdim) * (gate * torch.sigmoid(gate))) @ W[f"{prefix}.o"].T), S
 
 
 def feed_forward(h, prefix, W):
-    return (gelu_tanh(h @ W[f"{prefix}.gate"].T) * (h @ W[f"{prefix}.up"].T)) @ W[f"{prefix}.down"].T
+    return _r(_r(gelu_tanh(_r(h @ W[f"{prefix}.gate"].T)) * _r(h @ W[f"{prefix}.up"].T)) @ W[f"{prefix}.down"].T)
 
 
 def layer(x, index, W, entry, eps):
     prefix = f"l{index}"
     norm = lambda rows, name: layer_norm(rows, W[f"{prefix}.{name}"], W[f"{prefix}.{name}.b"], eps)
-    h = norm(x, "norm1")
+    h = _r(norm(x, "norm1"))
     mixer = entry["mixer"]
     if entry["type"] == "attention":
         mixed = sigmoid_attention(h, f"{prefix}.mix", W, mixer)
@@ -129,7 +159,7 @@ def layer(x, index, W, entry, eps):
         mixed = mixer.get("left_scale", 1.0) * left + mixer.get("right_scale", 1.0) * right
     x = x + norm(mixed, "norm1b")
     if entry.get("mlp") is not None:
-        x = x + norm(feed_forward(norm(x, "norm2"), f"{prefix}.mlp", W), "norm2b")
+        x = x + norm(feed_forward(_r(norm(x, "norm2")), f"{prefix}.mlp", W), "norm2b")
     return x
 
 
@@ -152,11 +182,11 @@ def forward(tokens, tensors, raw, stream_after=None):
     embedded = x
     for index, begins in run_order(raw):
         if begins is not None:
-            x = torch.cat([x, embedded], dim=-1) @ W["loop.in"].T + W["loop.step"][begins]
+            x = _r(torch.cat([x, embedded], dim=-1)) @ W["loop.in"].T + W["loop.step"][begins]
         x = layer(x, index, W, raw["layers"][index], eps)
         if stream_after is not None:
             stream_after.append(x)
-    x = layer_norm(x, W["final.norm"], W["final.norm.b"], eps)
+    x = _r(layer_norm(x, W["final.norm"], W["final.norm.b"], eps))
     return x @ W["head"].T * raw.get("logit_scale", 1.0)
 
 
@@ -167,3 +197,15 @@ def greedy(tokens, tensors, raw, count):
         out.append(int(forward(tokens, tensors, raw)[-1].argmax()))
         tokens.append(out[-1])
     return out
+
+
+def rounding_noise(tokens, tensors, raw, want, samples=8):
+    """Per position, the largest departure (max over the vocabulary) from ``want`` (the exact logits) among
+    ``samples`` runs with bfloat16-rounded activations: the first rounds to nearest, the others dither."""
+    generator = torch.Generator().manual_seed(1)
+    worst = torch.zeros(len(tokens), dtype=F64)
+    for sample in range(samples):
+        with activations_rounded_to(torch.bfloat16, generator if sample else None):
+            noisy = forward(tokens, tensors, raw)
+        worst = torch.maximum(worst, (noisy - want).abs().max(dim=-1).values)
+    return worst
