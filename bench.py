@@ -4,7 +4,7 @@ MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
     python bench.py --workload serving [--shape 0.5b|7b|34b]
     python bench.py --microbench
-    python bench.py --design mukutar|lutosun [--shape 0.5b|7b] [--layers L] [--window W] [--only mukutar|lutosun|falcon_h1]
+    python bench.py --design mukutar|lutosun|motolix [--shape 0.5b|7b] [--layers L] [--window W] [--only DESIGN|falcon_h1]
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
@@ -31,7 +31,10 @@ sizes are those of ``--shape``, and beside it the Falcon-H1 shape with the same 
 feed-forward width: for both the 2,048-token prompt step and decode steps at batch 1, 8 and 64 behind
 2,048-token contexts, each with its fraction of the peak (prompt: flops; decode: bytes the step has to read).
 ``--design lutosun`` does the same for a Lutosun-shaped model (latent attention, a routed mixture of experts beside
-a shared one, layer norms, a hashed bigram embedding).  The default workload and its line are not touched by either.
+a shared one, layer norms, a hashed bigram embedding), and ``--design motolix`` for a Motolix-shaped one (two layers
+in three softmax attention with normed projections and turned values beside gated linear attention, the third sigmoid
+attention whose values are its keys; a norm before and behind every branch; GELU-gated feed-forwards; the middle
+third of the layers run twice).  The default workload and its line are not touched by any of them.
 
 ``--workload serving`` runs whole requests through the scheduler and the sampler instead
 (``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
@@ -168,11 +171,38 @@ def lutosun_shape(shape: dict, layers: int) -> dict:
             "logit_softcap": 30.0, "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
 
 
+def motolix_shape(shape: dict, layers: int) -> dict:
+    """A Motolix configuration with the sizes of a Falcon-H1 ``shape``: the same width, vocabulary, feed-forward
+    width, attention heads and head size (values of the softmax side a quarter wider than its keys); the gated
+    linear side half as wide as the stream in keys and as wide as it in values.  ``layers`` counts runs: the
+    middle third of the layers runs twice."""
+    width, dim = shape["hidden_size"], shape["head_dim"]
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    sigmoid = {"type": "attention", "mixer": {
+        "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+        "rot": {"base": 5e5, "dims": dim // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    linear_heads = max(width // (2 * dim), 1)
+    parallel = {"type": "parallel", "mixer": {
+        "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim + dim // 4, "scale": dim ** -0.5,
+                 "rot": {"base": 5e5, "dims": dim}},
+        "right": {"heads": linear_heads, "dim": dim, "vdim": 2 * dim, "tau": 16.0},
+        "left_scale": 1.0, "right_scale": 1.0}}
+    kinds = (parallel, parallel, sigmoid)
+    mlp = {"kind": "dense", "ff": shape["intermediate_size"]}
+    looped = max(layers // 4, 1)                 # stored layers = runs - looped
+    stored = max(layers - looped, 2)
+    start = (stored - looped) // 2
+    return {"architecture": "Motolix", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
+            "embedding": {"scale": float(width) ** 0.5}, "logit_scale": 1.0,
+            "loop": {"start": start, "stop": start + looped, "times": 2},
+            "layers": [dict(kinds[index % 3], mlp=mlp) for index in range(stored)]}
+
+
 def design_points(args) -> int:
     """Prompt and decode steps of a model of another design with the sizes of a Falcon-H1 shape, and of that shape."""
     import torch
     from macllm_infer_amd import Engine, Lane
-    from macllm_infer_amd.config import FalconH1Config, LutosunConfig, MukutarConfig
+    from macllm_infer_amd.config import FalconH1Config, LutosunConfig, MotolixConfig, MukutarConfig
     from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
     from macllm_infer_amd.weights.random_init import random_tensors
 
@@ -182,6 +212,8 @@ def design_points(args) -> int:
     element = 2 if args.dtype == "bf16" else 4
     if args.design == "lutosun":
         configs = {"lutosun": LutosunConfig.from_dict(lutosun_shape(shape, layers))}
+    elif args.design == "motolix":
+        configs = {"motolix": MotolixConfig.from_dict(motolix_shape(shape, layers))}
     else:
         configs = {"mukutar": MukutarConfig.from_dict(mukutar_shape(shape, layers, args.window))}
     configs["falcon_h1"] = FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))
@@ -336,11 +368,11 @@ def main() -> int:
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     parser.add_argument("--microbench", action="store_true",
                         help="only this GPU's streaming read and read-modify-write bandwidth")
-    parser.add_argument("--design", default=None, choices=["mukutar", "lutosun"],
+    parser.add_argument("--design", default=None, choices=["mukutar", "lutosun", "motolix"],
                         help="measure a model of this design with the sizes of --shape (12 layers unless --layers) beside "
                              "the Falcon-H1 shape of equal sizes, instead of the headline workload")
     parser.add_argument("--window", type=int, default=1024, help="--design: the attention layers' window")
-    parser.add_argument("--only", default=None, choices=["mukutar", "lutosun", "falcon_h1"], help="--design: one of the two models")
+    parser.add_argument("--only", default=None, choices=["mukutar", "lutosun", "motolix", "falcon_h1"], help="--design: one of the two models")
     parser.add_argument("--write-config", default=None, metavar="PATH",
                         help="write the config.json of --shape / --layers there and exit (what "
                              "utils.kernel_trace --config reads)")
@@ -357,6 +389,8 @@ def main() -> int:
                 json.dump(mukutar_shape(shape, args.layers or 12, args.window), handle)
             elif args.design == "lutosun" and args.only != "falcon_h1":
                 json.dump(lutosun_shape(shape, args.layers or 12), handle)
+            elif args.design == "motolix" and args.only != "falcon_h1":
+                json.dump(motolix_shape(shape, args.layers or 12), handle)
             else:
                 layers = args.layers or (12 if args.design else shape["num_hidden_layers"])
                 json.dump(dict(shape, num_hidden_layers=layers), handle)

@@ -1128,15 +1128,21 @@ extern "C" int mi_decode_attention_static(const void* q, long q_ld, int T, int H
 
 // EXTRAS: the scores lose log_bias[head] = (r1, r2) -> r1 * ln(1 + r2 * distance), and the softmax's denominator
 // holds one more term exp(sinks[head]) (either pointer may be null).
-template <int DH, int NSET, bool EXTRAS = false>
+// DV: the width the values are computed with, the keys' or, PADDED, the next width of the launch's table above
+// value_dim, the width of the cached values and of a head's output (a multiple of 4).
+// SIGMOID: a visible key weighs sigmoid(score * scale * head_scales[head] + score_bias[head]) on its own (either
+// pointer may be null: 1 and 0); no maximum, no normalizer, the waves' partial sums are added as they are.
+template <int DH, int NSET, bool EXTRAS = false, int DV = DH, bool SIGMOID = false, bool PADDED = false>
 __global__ void __launch_bounds__(PREFILL_WAVES * WAVE)
 prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hkv, const bf16_t* __restrict__ k_base,
                          const bf16_t* __restrict__ v_base, long page_stride, int page_size,
                          const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale,
                          int window, bf16_t* __restrict__ out, long out_ld,
-                         const float* __restrict__ log_bias = nullptr, const float* __restrict__ sinks = nullptr) {
-  constexpr int ITEMS = 2 + 4 * (DH / 16);                    // m, l and the accumulator of one set
+                         const float* __restrict__ log_bias = nullptr, const float* __restrict__ sinks = nullptr,
+                         int value_dim = DV, const float* __restrict__ head_scales = nullptr,
+                         const float* __restrict__ score_bias = nullptr) {
+  constexpr int ITEMS = 2 + 4 * (DV / 16);                    // m, l and the accumulator of one set
   __shared__ float part[PREFILL_WAVES][ITEMS][WAVE];
   __shared__ int wave_pages[PREFILL_WAVES][WAVE];
   // heavy ones first; every other head pass the other way round, so that workgroups of two passes that
@@ -1181,8 +1187,17 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
       }
     }
   }
-  AttnAccumulator<DH, NSET> acc;
+  AttnAccumulator<DH, NSET, DV> acc;
   acc.clear();
+  AttnGate<NSET> gate;
+  if (SIGMOID) {
+#pragma unroll
+    for (int s = 0; s < NSET; ++s) {
+      const int head = min(head0 + s, Hq - 1);
+      gate.scale[s] = scale * (head_scales ? head_scales[head] : 1.f);
+      gate.bias[s] = score_bias ? score_bias[head] : 0.f;
+    }
+  }
   AttnLogBias<NSET> bias;
   if (EXTRAS) {
     bias.on = log_bias != nullptr;
@@ -1199,6 +1214,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   cache.page_stride = page_stride;
   cache.page_size = page_size;
   cache.kvh = kvh;
+  cache.value_dim = value_dim;
   const int* cache_pages = block_tables + (long)request * max_pages;
   int key_lo = 0;
   if (window > 0 && first_position - window + 1 > 0) key_lo = ((first_position - window + 1) / 32) * 32;
@@ -1215,8 +1231,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
     cache.pages = wave_pages[wave];
     cache.base_page = first_page;
-    attend_keys<DH, NSET, PREFILL_STEPS, false, EXTRAS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache,
-                                                        full_tile ? first_position : -1, last_position, bias);
+    attend_keys<DH, NSET, PREFILL_STEPS, false, EXTRAS, DV, SIGMOID, PADDED>(
+        acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache, full_tile ? first_position : -1, last_position,
+        bias, &gate);
     part_lo = part_hi;
   }
 
@@ -1227,11 +1244,28 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     part[wave][0][lane] = acc.m[s];
     part[wave][1][lane] = acc.l[s];
 #pragma unroll
-    for (int dt = 0; dt < DH / 16; ++dt)
+    for (int dt = 0; dt < DV / 16; ++dt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) part[wave][2 + 4 * dt + i][lane] = acc.o[s][dt][i];
     __syncthreads();
     if (wave != s % PREFILL_WAVES) continue;
+    if (SIGMOID) {
+      if (col_pos[s] < 0) continue;
+      bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * value_dim;
+#pragma unroll
+      for (int dt = 0; dt < DV / 16; ++dt) {
+        mfma_bf16x4 packed;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float value = 0.f;
+#pragma unroll
+          for (int w = 0; w < PREFILL_WAVES; ++w) value += part[w][2 + 4 * dt + i][lane];
+          packed[i] = (bf16_t)value;
+        }
+        if (!PADDED || 16 * dt + 4 * qd < value_dim) *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
+      }
+      continue;
+    }
     float m = -INFINITY;
 #pragma unroll
     for (int w = 0; w < PREFILL_WAVES; ++w) m = fmaxf(m, part[w][0][lane]);
@@ -1251,9 +1285,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     if (EXTRAS && sinks) l += __builtin_amdgcn_exp2f(sink - m);       // once for the column: no key, no value
     if (col_pos[s] < 0) continue;
     const float inverse = 1.f / l;
-    bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * DH;
+    bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * value_dim;
 #pragma unroll
-    for (int dt = 0; dt < DH / 16; ++dt) {
+    for (int dt = 0; dt < DV / 16; ++dt) {
       mfma_bf16x4 packed;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1262,9 +1296,69 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
         for (int w = 0; w < PREFILL_WAVES; ++w) value += part[w][2 + 4 * dt + i][lane] * factor[w];
         packed[i] = (bf16_t)(value * inverse);
       }
-      *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
+      if (!PADDED || 16 * dt + 4 * qd < value_dim) *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
     }
   }
+}
+
+// The widths the values are computed with when they are not the keys' (the cached width rounded up to one of them),
+// and the query heads that share a key fragment at that width: the accumulators of a set grow with it.
+static int padded_value_width(int dv) {
+  const int widths[] = {32, 64, 96, 128, 160, 192, 256};
+  for (int width : widths)
+    if (dv <= width) return width;
+  return 0;
+}
+
+// The same kernel for two further forms (bfloat16, head_dim 64 or 128):
+//   values of another width than the keys (dv a multiple of 4 up to 256; softmax, no window bias or sink), and
+//   sigmoid weights with a multiplier and a bias per head (either null), values as wide as the keys.
+// Returns ERR_UNSUPPORTED_SIZE for what it does not cover (the caller uses mi_paged_attention).
+extern "C" int mi_prefill_attention_forms(const void* q, long q_ld, int Hq, int Hkv, int dh, int dv, const void* k_base,
+                                          const void* v_base, long page_stride, int page_size,
+                                          const int* block_tables, int max_pages, const int* tiles, int n_tiles,
+                                          const int* cu_seqlens, const int* start_pos, float scale, int window,
+                                          int max_seq_len, void* out, long out_ld, int sigmoid,
+                                          const float* head_scales, const float* score_bias, hipStream_t stream) {
+  if (n_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || max_pages <= 0 || dv <= 0)
+    return ERR_BAD_ARGUMENT;
+  const int G = Hq / Hkv;
+  if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64 ||
+      dv % 4 != 0 || n_tiles > (1 << 28))
+    return ERR_UNSUPPORTED_SIZE;
+  if (sigmoid ? dv != dh : (dv == dh || head_scales || score_bias)) return ERR_UNSUPPORTED_SIZE;
+  const int width = sigmoid ? dh : padded_value_width(dv);
+  if (width == 0) return ERR_UNSUPPORTED_SIZE;
+  const int widest = width > dh ? width : dh;
+  int most = widest <= 64 ? 4 : widest <= 128 ? 2 : 1;
+  if (most > 2 && max_seq_len <= 2048 && 4L * n_tiles * Hkv * ((G + most - 1) / most) < PREFILL_FILL_BLOCKS) most = 2;
+  const int passes = (G + most - 1) / most;
+  const int nset = (G + passes - 1) / passes;
+  const dim3 grid(4 * n_tiles, Hkv, passes);
+#define FORM_ARGS                                                                                              \
+  (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size,       \
+      block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, nullptr,     \
+      nullptr, dv, head_scales, score_bias
+#define SIGMOID_CASE(DH_, NSET_)                                                                               \
+  if (sigmoid && dh == DH_ && nset == NSET_)                                                                   \
+    prefill_attention_kernel<DH_, NSET_, false, DH_, true, false><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(FORM_ARGS);
+#define PADDED_CASE(DH_, DV_, NSET_)                                                                           \
+  if (!sigmoid && dh == DH_ && width == DV_ && nset == NSET_)                                                  \
+    prefill_attention_kernel<DH_, NSET_, false, DV_, false, true><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(FORM_ARGS);
+  SIGMOID_CASE(64, 1) SIGMOID_CASE(64, 2) SIGMOID_CASE(64, 3) SIGMOID_CASE(64, 4)
+  SIGMOID_CASE(128, 1) SIGMOID_CASE(128, 2)
+  PADDED_CASE(64, 32, 1) PADDED_CASE(64, 32, 2) PADDED_CASE(64, 32, 3) PADDED_CASE(64, 32, 4)
+  PADDED_CASE(64, 64, 1) PADDED_CASE(64, 64, 2) PADDED_CASE(64, 64, 3) PADDED_CASE(64, 64, 4)
+  PADDED_CASE(64, 96, 1) PADDED_CASE(64, 96, 2) PADDED_CASE(64, 128, 1) PADDED_CASE(64, 128, 2)
+  PADDED_CASE(64, 160, 1) PADDED_CASE(64, 192, 1) PADDED_CASE(64, 256, 1)
+  PADDED_CASE(128, 32, 1) PADDED_CASE(128, 32, 2) PADDED_CASE(128, 64, 1) PADDED_CASE(128, 64, 2)
+  PADDED_CASE(128, 96, 1) PADDED_CASE(128, 96, 2) PADDED_CASE(128, 128, 1) PADDED_CASE(128, 128, 2)
+  PADDED_CASE(128, 160, 1) PADDED_CASE(128, 192, 1) PADDED_CASE(128, 256, 1)
+#undef SIGMOID_CASE
+#undef PADDED_CASE
+#undef FORM_ARGS
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
 }
 
 // tiles: int32 [n_tiles, 2] = (lane, first token row of the tile); a tile never crosses a lane.

@@ -50,6 +50,7 @@ struct AttnCache {
   int kvh;
   const int* pages;      // page id of logical page (index + base_page); LDS or global
   int base_page;
+  int value_dim;         // PADDED loads only: the width of a cached value, at most the DV the wave computes with
 };
 
 // The K and V fragments of STEPS steps of 32 keys from key k00 on.  K: rows of two 16-key tiles
@@ -61,7 +62,9 @@ struct AttnFragments {
   mfma_bf16x8 v[STEPS][DV / 16];
 };
 
-template <int DH, int STEPS, int DV = DH>
+// PADDED: the cached values are cache.value_dim wide, less than DV; the rows past them repeat the last one (their
+// results are never stored).
+template <int DH, int STEPS, int DV = DH, bool PADDED = false>
 __device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS, DV>& f, int k00, int last_key, const AttnCache& cache) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int q = lane / 16;
@@ -89,9 +92,10 @@ __device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS, DV>& f, int k
     for (int dt = 0; dt < DV / 16; ++dt) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
+        const long value_row = PADDED ? (long)cache.kvh * cache.value_dim + min(16 * dt + r, cache.value_dim - 1)
+                                      : (long)cache.kvh * DV + 16 * dt + r;
         const mfma_bf16x4 part = *reinterpret_cast<const mfma_bf16x4*>(
-            cache.v_base + (long)page[t] * cache.page_stride +
-            ((long)cache.kvh * DV + 16 * dt + r) * cache.page_size + offset[t]);
+            cache.v_base + (long)page[t] * cache.page_stride + value_row * cache.page_size + offset[t]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) f.v[st][dt][4 * t + j] = part[j];
       }
@@ -109,15 +113,25 @@ struct AttnLogBias {
   float r2[NSET];
 };
 
+// Weights that are no softmax: a visible key weighs sigmoid(score * scale[set] + bias[set]) on its own, one pair
+// of numbers for each set of columns (a query head); nothing is normalized, the accumulator is a plain sum.
+template <int NSET>
+struct AttnGate {
+  float scale[NSET];
+  float bias[NSET];
+};
+
 // Scores, softmax step and values of the loaded steps, per set of columns.
 // MASKED = false: the caller vouches that every key of the round is visible to every column
 // and lies inside the run (steps away from the diagonal, the window's edge and the run's end):
 // no masks are computed.
-template <int DH, int NSET, int STEPS, bool MASKED = true, bool BIASED = false, int DV = DH>
+// SIGMOID: the weights of ``gate`` instead of the softmax (acc.m and acc.l stay as they were cleared).
+template <int DH, int NSET, int STEPS, bool MASKED = true, bool BIASED = false, int DV = DH, bool SIGMOID = false>
 __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc, AttnFragments<DH, STEPS, DV>& f,
                                              const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                              const int (&col_pos)[NSET], int window, float scale, int k00,
-                                             int key_hi, const AttnLogBias<NSET>& bias = AttnLogBias<NSET>()) {
+                                             int key_hi, const AttnLogBias<NSET>& bias = AttnLogBias<NSET>(),
+                                             const AttnGate<NSET>* gate = nullptr) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int q = lane / 16;
   const int last_key = key_hi - 1;
@@ -183,6 +197,24 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
             score[t][i] = visible ? score[t][i] : -INFINITY;
           }
       }
+      if (SIGMOID) {
+        // 1 / (1 + exp(-(s * scale + bias))) with the exponent in units of log2; a masked score of -inf gives 0
+        const float slope = -gate->scale[s] * 1.4426950408889634f;
+        const float offset = -gate->bias[s] * 1.4426950408889634f;
+        mfma_bf16x8 p_frag;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = score[t][i] == -INFINITY ? 0.f
+                                                     : 1.f / (1.f + __builtin_amdgcn_exp2f(fmaf(score[t][i], slope, offset)));
+            p_frag[4 * t + i] = (bf16_t)p;
+          }
+#pragma unroll
+        for (int dt = 0; dt < DV / 16; ++dt)
+          acc.o[s][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[st][dt], p_frag, acc.o[s][dt], 0, 0, 0);
+        continue;
+      }
       float step_max = fmaxf(fmaxf(fmaxf(score[0][0], score[0][1]), fmaxf(score[0][2], score[0][3])),
                              fmaxf(fmaxf(score[1][0], score[1][1]), fmaxf(score[1][2], score[1][3])));
       step_max = fmaxf(step_max, __shfl_xor(step_max, 16, WAVE));
@@ -222,12 +254,15 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
 // with long runs; a caller whose run is one round of STEPS steps gains nothing from it.
 // min_pos / max_pos: the smallest and largest position among the columns of the wave, when all
 // of them hold queries and the caller knows (the same value in every lane), else -1.
-template <int DH, int NSET, int STEPS, bool PIPELINED = false, bool BIASED = false, int DV = DH>
+// SIGMOID (with ``gate``) and PADDED (with cache.value_dim): see attn_compute and attn_load; not PIPELINED.
+template <int DH, int NSET, int STEPS, bool PIPELINED = false, bool BIASED = false, int DV = DH, bool SIGMOID = false,
+          bool PADDED = false>
 __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET, DV>& acc,
                                             const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                             const int (&col_pos)[NSET], int window, float scale, int key_lo,
                                             int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1,
-                                            const AttnLogBias<NSET>& bias = AttnLogBias<NSET>()) {
+                                            const AttnLogBias<NSET>& bias = AttnLogBias<NSET>(),
+                                            const AttnGate<NSET>* gate = nullptr) {
   const int last_key = key_hi - 1;
   constexpr int ROUND = 32 * STEPS;
   if (PIPELINED) {
@@ -250,13 +285,15 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET, DV>& acc,
       open_hi = key_lo + max(0, (min(min_pos + 1, key_hi) - key_lo) / ROUND) * ROUND;
     for (int k00 = key_lo; k00 < open_hi; k00 += ROUND) {
       AttnFragments<DH, STEPS, DV> f;
-      attn_load<DH, STEPS, DV>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, false, BIASED, DV>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
+      attn_load<DH, STEPS, DV, PADDED>(f, k00, last_key, cache);
+      attn_compute<DH, NSET, STEPS, false, BIASED, DV, SIGMOID>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias,
+                                                                gate);
     }
     for (int k00 = open_hi; k00 < key_hi; k00 += ROUND) {
       AttnFragments<DH, STEPS, DV> f;
-      attn_load<DH, STEPS, DV>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, true, BIASED, DV>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
+      attn_load<DH, STEPS, DV, PADDED>(f, k00, last_key, cache);
+      attn_compute<DH, NSET, STEPS, true, BIASED, DV, SIGMOID>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias,
+                                                               gate);
     }
   }
 }

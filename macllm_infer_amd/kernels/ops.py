@@ -103,6 +103,9 @@ _SIGNATURES = {
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
                                  _c_ptr, _c_ptr, _c_ptr],
+        "mi_prefill_attention_forms": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
+                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr,
+                                       _c_long, _c_int, _c_ptr, _c_ptr, _c_ptr],
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_long, _c_ptr],
@@ -1112,6 +1115,54 @@ def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
         _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, _p(log_bias),
         _p(sinks), _stream()), "prefill_attention")
+
+
+PREFILL_VALUE_WIDTH_MOST = 256      # the widest values the matrix-core kernel computes with
+
+
+def prefill_attention_forms_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                                      page_size: int, sigmoid: bool, per_head: bool) -> bool:
+    """Whether the matrix-core kernel's further forms cover this: sigmoid weights (with a multiplier and a bias per
+    head, ``per_head``) over values as wide as the keys, or a softmax over values of another width."""
+    if not (dtype == torch.bfloat16 and head_dim in (64, 128) and page_size % 4 == 0
+            and num_heads // num_kv_heads <= 64 and value_dim % 4 == 0):
+        return False
+    if sigmoid:
+        return value_dim == head_dim
+    return value_dim != head_dim and value_dim <= PREFILL_VALUE_WIDTH_MOST and not per_head
+
+
+def prefill_attention_forms(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                            k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                            query_tiles: torch.Tensor, cu_seqlens: torch.Tensor, start_pos: torch.Tensor, scale: float,
+                            window: Optional[int], out: torch.Tensor, max_seq_len: int = 0, sigmoid: bool = False,
+                            head_scales: Optional[torch.Tensor] = None, score_bias: Optional[torch.Tensor] = None) -> None:
+    """``prefill_attention`` for values of another width than the keys (``out`` [T, Hq * value_dim]), or, with
+    ``sigmoid``, for weights sigmoid(score * scale * head_scales[h] + score_bias[h]) that are not normalized."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "prefill_attention_forms: bfloat16 only")
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * value_dim) and q_ld % 8 == 0
+          and q.data_ptr() % 16 == 0 and out_ld % 4 == 0 and out.data_ptr() % 8 == 0,
+          "prefill_attention_forms: q/out shapes or alignment do not fit")
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype, value_dim)
+    _need(prefill_attention_forms_supported(q.dtype, num_heads, num_kv_heads, head_dim, value_dim, page_size, sigmoid,
+                                            head_scales is not None or score_bias is not None),
+          "prefill_attention_forms: not covered; use paged_attention")
+    for name, tensor in (("block_tables", block_tables), ("query_tiles", query_tiles), ("cu_seqlens", cu_seqlens),
+                         ("start_pos", start_pos)):
+        _i32(tensor, name)
+    _need(block_tables.dim() == 2 and query_tiles.dim() == 2 and query_tiles.shape[1] == 2
+          and cu_seqlens.numel() == start_pos.numel() + 1, "prefill_attention_forms: metadata shapes do not match")
+    for name, tensor in (("head_scales", head_scales), ("score_bias", score_bias)):
+        _need(tensor is None or (tensor.dtype == torch.float32 and tensor.numel() == num_heads and tensor.is_contiguous()
+                                 and tensor.is_cuda), f"prefill_attention_forms: {name} must be float32 [Hq] on the GPU")
+    _check(_fn("attention", "mi_prefill_attention_forms")(
+        _p(q), q_ld, num_heads, num_kv_heads, head_dim, int(value_dim), _p(k_cache), _p(v_cache), page_stride,
+        page_size, _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
+        _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, 1 if sigmoid else 0,
+        _p(head_scales), _p(score_bias), _stream()), "prefill_attention_forms")
 
 
 def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:

@@ -233,6 +233,14 @@ class Attention(Mixer):
             ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                   step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window, out,
                                   step.max_seq_len)
+        elif (tiles and aligned and step.query_tile == self.query_tile
+                and ops.prefill_attention_forms_supported(qkv.dtype, *geometry, spec.value_width, cache.k_cache.shape[2],
+                                                          sigmoid, self.head_scales is not None)):
+            # the matrix-core kernel's further forms: sigmoid weights, or values of another width than the keys
+            ops.prefill_attention_forms(qkv, *geometry, spec.value_width, cache.k_cache, cache.v_cache,
+                                        step.block_tables[cache.group], step.query_tiles, step.cu_seqlens,
+                                        step.start_pos, spec.scale, spec.window, out, step.max_seq_len, sigmoid=sigmoid,
+                                        head_scales=self.head_scales, score_bias=self.score_bias)
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, out, step.max_seq_len,

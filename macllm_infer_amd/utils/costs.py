@@ -44,7 +44,11 @@ def model_sizes(spec) -> dict:
             if part.kind == "attention":
                 q, kv = part.num_heads * part.head_dim, part.num_kv_heads * part.head_dim
                 values, mixed = part.num_kv_heads * part.value_width, part.num_heads * part.value_width
-                total["in_weights"] += (q + kv + values) * d
+                # values that are the keys as projected have no matrix of their own, but cells of their own in the cache
+                projected = 0 if getattr(part, "values_from_keys", False) else values
+                if getattr(part, "projection_norm_eps", None) is not None:
+                    total["in_weights"] += q + kv                          # the norms' weights over whole projections
+                total["in_weights"] += (q + kv + projected) * d
                 total["out_weights"] += d * mixed
                 total["kv_per_token"] += kv + values if entry.kv_from is None else 0
                 # x 2 T^2 flops (causal: half of 4 T^2); a window w keeps min(i + 1, w) keys for the query at i
@@ -52,7 +56,16 @@ def model_sizes(spec) -> dict:
                 total["windows"].append((part.num_heads * (part.head_dim + part.value_width) / 2.0,
                                          (kv + values) if entry.kv_from is None else 0, part.window))
                 total["mixed"] += mixed
-                total["in_width"] += q + kv + values
+                total["in_width"] += q + kv + projected
+            elif part.kind == "gated_linear_attention":
+                keys, values = part.num_heads * part.key_dim, part.num_heads * part.value_dim
+                rank = part.decay_rank or 16
+                total["in_weights"] += (2 * keys + 2 * values + rank) * d + keys * rank
+                total["out_weights"] += d * values
+                total["state"] += part.num_heads * part.key_dim * part.value_dim
+                total["linear_scan"] += 5 * part.num_heads * part.key_dim * part.value_dim     # x T flops
+                total["mixed"] += values
+                total["in_width"] += 2 * keys + 2 * values + rank + 2 * keys                  # the decays in float32
             elif part.kind == "latent_attention":
                 heads, rank, turned = part.num_heads, part.kv_rank, part.rope_dim
                 q = heads * (part.head_dim + turned)
@@ -90,6 +103,8 @@ def model_sizes(spec) -> dict:
                 total["scan"] += part.num_heads * part.head_dim * part.state_size      # x 6 T flops
                 total["mixed"] += part.inner_size
                 total["in_width"] += part.projection_width
+        if entry.before is not None and getattr(entry.before, "mix_name", None) is not None:
+            total["in_weights"] += 2 * d * d                               # the stream mixed with the embedding output
         if layer.ffn is None:
             continue
         if layer.ffn.kind == "swiglu":
@@ -184,7 +199,7 @@ def total(costs: Dict[str, Cost]) -> Cost:
 DECODE_GROUPS: List[Tuple[str, str]] = [
     (r"mixer_decode_kernel|mixer_merge_kernel|decode_attention_kernel|decode_merge_kernel|ssm_scan_kernel|conv_step_kernel|"
      r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel|paged_attention_tile_kernel|"
-     r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel|latent_|rotate_heads_kernel", "mixers"),
+     r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel|latent_|rotate_heads_kernel|attention_prepare_kernel", "mixers"),
     (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
     (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1|moe_|clamped_glu_kernel", "gate and up projections"),
     (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
@@ -194,7 +209,7 @@ PLAIN_PRODUCT = r"fused_gemm_kernel<\d+, [01], 0"
 PREFILL_GROUPS: List[Tuple[str, str]] = [
     (r"^Cijk_|gemm_f32_kernel|head_gemm_kernel|moe_expert_gemm", "matrix products"),
     (r"prefill_attention|paged_attention_kernel|paged_attention_tile_kernel|paged_attention_merge_kernel|"
-     r"rope_kv_store_kernel|latent_", "attention"),
+     r"rope_kv_store_kernel|latent_|attention_prepare_kernel|rotate_heads_kernel", "attention"),
     (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel|linear_state_|head_norm_gate_kernel|"
      r"tanh_rows_kernel", "state-space scan"),
 ]

@@ -101,7 +101,8 @@ def sigmoid_spec(H, G, D, scale, rotation):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H, G, D, rot_dims, scaling", [
     (6, 2, 16, 16, None), (3, 3, 24, 12, (8.0, 1.0, 4.0, 64)), (4, 2, 64, 32, (2.0, 1.0, 4.0, 512)),
-    (2, 2, 128, 128, None), (5, 1, 8, 2, None), (1, 1, 80, 80, (16.0, 2.0, 8.0, 128))])
+    (2, 2, 128, 128, None), (5, 1, 8, 2, None), (1, 1, 80, 80, (16.0, 2.0, 8.0, 128)),
+    (8, 1, 64, 64, None), (3, 1, 128, 64, None), (10, 2, 64, 16, None)])
 def test_sigmoid_attention_alone(dtype, H, G, D, rot_dims, scaling):
     hidden = 40
     rotation = motolix_configs.rot(700.0, rot_dims, scaling)
@@ -192,7 +193,8 @@ def softmax_spec(H, G, D, V, scale, rotation):
 @pytest.mark.parametrize("H, G, D, V, rot_dims, scaling", [
     (6, 2, 16, 16, 16, None), (3, 3, 24, 40, 12, None), (4, 1, 64, 64, 64, (4.0, 1.0, 4.0, 128)),
     (6, 2, 64, 80, 32, None), (2, 2, 128, 128, 128, None), (5, 1, 8, 24, 4, None), (2, 1, 48, 6, 48, None),
-    (4, 2, 64, 128, 64, None)])
+    (4, 2, 64, 128, 64, None), (2, 1, 128, 160, 64, None), (3, 1, 64, 32, 64, None), (8, 1, 64, 96, 32, None),
+    (5, 1, 128, 72, 128, None), (1, 1, 64, 256, 64, None), (3, 1, 128, 12, 32, None), (2, 2, 64, 200, 64, None)])
 def test_softmax_attention_with_normed_projections_and_turned_values_alone(dtype, H, G, D, V, rot_dims, scaling):
     hidden = 40
     rotation = motolix_configs.rot(3000.0, rot_dims, scaling)
@@ -217,6 +219,47 @@ def test_the_projection_norm_runs_over_all_heads_at_once():
     harness = PartHarness(softmax_spec(H, G, D, V, 1.5, rotation), tensors, hidden, torch.float32, page_size=8)
     got = torch.cat([harness.run([("r", x[:50])])[0]] + [harness.run([("r", x[t:t + 1])])[0] for t in range(50, 70)])
     close(got, want, torch.float32, "norm over the whole projection")
+
+
+@pytest.mark.parametrize("sigmoid, H, G, D, V", [(True, 4, 2, 64, 64), (True, 2, 1, 128, 128), (False, 6, 2, 64, 80),
+                                                 (False, 2, 1, 128, 160), (False, 4, 4, 64, 32)])
+def test_prompt_portions_in_bfloat16_run_on_the_matrix_cores(monkeypatch, sigmoid, H, G, D, V):
+    """Heads of 64 and 128 in bfloat16: portions of prompts (alone and beside single tokens) go through the
+    matrix-core kernel's forms for sigmoid weights and for values of another width than the keys, single tokens
+    through the general kernel; both against the plain model, and each is seen to have run."""
+    from macllm_infer_amd.kernels import ops
+    calls = {"forms": 0, "general": 0}
+    forms, general = ops.prefill_attention_forms, ops.paged_attention
+
+    def spy_forms(*args, **more):
+        calls["forms"] += 1
+        return forms(*args, **more)
+
+    def spy_general(*args, **more):
+        calls["general"] += 1
+        return general(*args, **more)
+    monkeypatch.setattr(ops, "prefill_attention_forms", spy_forms)
+    monkeypatch.setattr(ops, "paged_attention", spy_general)
+    hidden, dtype = 64, torch.bfloat16
+    rotation = motolix_configs.rot(2000.0, D // 2)
+    x = rand(200, hidden, seed=11).to(dtype).float()
+    if sigmoid:
+        tensors = rounded(sigmoid_tensors(hidden, H, G, D, seed=V), dtype)
+        mixer = {"heads": H, "kv_heads": G, "dim": D, "scale": 1.0 / math.sqrt(D), "rot": rotation}
+        want = motolix_plain.sigmoid_attention(x.double(), "p", stored(tensors), mixer)
+        spec = sigmoid_spec(H, G, D, mixer["scale"], rotation)
+    else:
+        tensors = rounded(softmax_tensors(hidden, H, G, D, V, seed=V), dtype)
+        mixer = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": 3.0 / math.sqrt(D), "rot": rotation}
+        want = motolix_plain.softmax_attention(x.double(), "p", stored(tensors), mixer, EPS)
+        spec = softmax_spec(H, G, D, V, mixer["scale"], rotation)
+    harness = PartHarness(spec, tensors, hidden, dtype, page_size=16)
+    first, = harness.run([("r", x[:70])])
+    second, _ = harness.run([("r", x[70:199]), ("other", x[:1])])
+    assert calls == {"forms": 2, "general": 0}
+    last, = harness.run([("r", x[199:])])
+    assert calls == {"forms": 2, "general": 1}
+    close(torch.cat([first, second, last]), want, dtype, "portions on the matrix cores")
 
 
 def crafted_softmax(distance, length, V=8):
