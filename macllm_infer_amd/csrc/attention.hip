@@ -830,6 +830,10 @@ struct alignas(16) bf16x8 {
   bf16_t v[8];
 };
 
+// dv: the width of a value head and of a head's output (any width; the keys' when it is DH).  head_scales
+// (a multiplier on a head's scores, after `scale`) and score_bias may be null.  sigmoid: a visible key weighs
+// sigmoid(score + score_bias[head]) on its own; the block then records (0, 1) as its (max, sum) and the merge adds
+// the partial outputs as they are.  Dynamic LDS: DEC_WAVES * G * dv floats.
 template <int DH, int G>
 __global__ void __launch_bounds__(DEC_THREADS)
 decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const bf16_t* __restrict__ k_base,
@@ -837,14 +841,14 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
                         const int* __restrict__ block_tables, int max_pages,
                         const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
                         int window, int split_keys, int splits, float* __restrict__ partial_o,
-                        float* __restrict__ partial_ml) {
+                        float* __restrict__ partial_ml, int dv, const float* __restrict__ head_scales,
+                        const float* __restrict__ score_bias, int sigmoid) {
   constexpr int LPR = DH / 8;
   constexpr int KPW = WAVE / LPR;
   constexpr int KPB = KPW * DEC_WAVES;
-  constexpr int DPL = DH / WAVE;
   __shared__ float s_lds[G][DEC_MAX_SPLIT];
   __shared__ float red[DEC_WAVES][G];
-  __shared__ float acc_lds[DEC_WAVES][G][DH];
+  extern __shared__ float acc_lds[];             // [DEC_WAVES][G][dv]
 
   const int split = blockIdx.x;
   const int kvh = blockIdx.y;
@@ -864,11 +868,14 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
   const int c = lane % LPR;
 
   float qf[G][8];
+  float offset_of[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const bf16x8 packed = *reinterpret_cast<const bf16x8*>(q + token * q_ld + (long)(kvh * G + g) * DH + c * 8);
+    const float factor = head_scales ? scale * head_scales[kvh * G + g] : scale;
+    offset_of[g] = score_bias ? score_bias[kvh * G + g] : 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) qf[g][j] = (float)packed.v[j] * scale;
+    for (int j = 0; j < 8; ++j) qf[g][j] = (float)packed.v[j] * factor;
   }
 
   // scores
@@ -898,89 +905,100 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
       for (int g = 0; g < G; ++g) s[g] += __shfl_xor(s[g], offset, WAVE);
     if (valid && c == 0) {
 #pragma unroll
-      for (int g = 0; g < G; ++g) s_lds[g][local] = key >= first_key ? s[g] : -INFINITY;
+      for (int g = 0; g < G; ++g) s_lds[g][local] = key >= first_key ? s[g] + offset_of[g] : -INFINITY;
     }
   }
   __syncthreads();
 
-  // softmax over the range: maximum, then exp and sum
   float m[G], l[G];
+  if (sigmoid) {
+    // every key on its own: 1 / (1 + exp(-s)); a key before the window's first (-inf) weighs nothing
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = -INFINITY;
-    for (int i = tid; i < count; i += DEC_THREADS) v = fmaxf(v, s_lds[g][i]);
-    v = wave_max(v);
-    if (lane == 0) red[wave][g] = v;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = red[0][g];
-#pragma unroll
-    for (int w = 1; w < DEC_WAVES; ++w) v = fmaxf(v, red[w][g]);
-    m[g] = v;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float sum = 0.f;
-    for (int i = tid; i < count; i += DEC_THREADS) {
-      const float p = __expf(s_lds[g][i] - m[g]);
-      s_lds[g][i] = p;
-      sum += p;
+    for (int g = 0; g < G; ++g) {
+      for (int i = tid; i < count; i += DEC_THREADS) {
+        const float score = s_lds[g][i];
+        s_lds[g][i] = score == -INFINITY ? 0.f : __builtin_amdgcn_rcpf(1.f + __expf(-score));
+      }
+      m[g] = 0.f;
+      l[g] = 1.f;
     }
-    sum = wave_sum(sum);
-    if (lane == 0) red[wave][g] = sum;
+  } else {
+    // softmax over the range: maximum, then exp and sum
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float v = -INFINITY;
+      for (int i = tid; i < count; i += DEC_THREADS) v = fmaxf(v, s_lds[g][i]);
+      v = wave_max(v);
+      if (lane == 0) red[wave][g] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float v = red[0][g];
+#pragma unroll
+      for (int w = 1; w < DEC_WAVES; ++w) v = fmaxf(v, red[w][g]);
+      m[g] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float sum = 0.f;
+      for (int i = tid; i < count; i += DEC_THREADS) {
+        const float p = __expf(s_lds[g][i] - m[g]);
+        s_lds[g][i] = p;
+        sum += p;
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) red[wave][g] = sum;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < DEC_WAVES; ++w) v += red[w][g];
+      l[g] = v;
+    }
   }
   __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = 0.f;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) v += red[w][g];
-    l[g] = v;
-  }
 
-  // values: each wave takes every fourth page of the range
-  float acc[G][DPL];
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) acc[g][i] = 0.f;
+  // values: each wave takes every fourth page of the range, 64 dims of the value head at a time
   const int range_pages = (count + page_size - 1) / page_size;
-  for (int pg = wave; pg < range_pages; pg += DEC_WAVES) {
-    const int local0 = pg * page_size;
-    const int page = table[(range_lo + local0) / page_size];
-    const int keys_here = min(page_size, count - local0);
+  for (int dim0 = 0; dim0 < dv; dim0 += WAVE) {
+    const int dim = dim0 + lane;
+    float acc[G];
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      const int dim = lane + i * WAVE;
-      const bf16_t* v_row = v_base + (long)page * page_stride + ((long)kvh * DH + dim) * page_size;
-      for (int j0 = 0; j0 < keys_here; j0 += 8) {
-        const bf16x8 packed = *reinterpret_cast<const bf16x8*>(v_row + j0);
+    for (int g = 0; g < G; ++g) acc[g] = 0.f;
+    if (dim < dv) {
+      for (int pg = wave; pg < range_pages; pg += DEC_WAVES) {
+        const int local0 = pg * page_size;
+        const int page = table[(range_lo + local0) / page_size];
+        const int keys_here = min(page_size, count - local0);
+        const bf16_t* v_row = v_base + (long)page * page_stride + ((long)kvh * dv + dim) * page_size;
+        for (int j0 = 0; j0 < keys_here; j0 += 8) {
+          const bf16x8 packed = *reinterpret_cast<const bf16x8*>(v_row + j0);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (j0 + j < keys_here) {
-            const float value = (float)packed.v[j];
+          for (int j = 0; j < 8; ++j) {
+            if (j0 + j < keys_here) {
+              const float value = (float)packed.v[j];
 #pragma unroll
-            for (int g = 0; g < G; ++g) acc[g][i] = fmaf(s_lds[g][local0 + j0 + j], value, acc[g][i]);
+              for (int g = 0; g < G; ++g) acc[g] = fmaf(s_lds[g][local0 + j0 + j], value, acc[g]);
+            }
           }
         }
       }
+#pragma unroll
+      for (int g = 0; g < G; ++g) acc_lds[((long)wave * G + g) * dv + dim] = acc[g];
     }
   }
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) acc_lds[wave][g][lane + i * WAVE] = acc[g][i];
   __syncthreads();
-  for (int index = tid; index < G * DH; index += DEC_THREADS) {
-    const int g = index / DH;
-    const int dim = index - g * DH;
+  for (int index = tid; index < G * dv; index += DEC_THREADS) {
+    const int g = index / dv;
+    const int dim = index - g * dv;
     float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) sum += acc_lds[w][g][dim];
-    partial_o[((token * Hq + kvh * G + g) * splits + split) * DH + dim] = sum;
+    for (int w = 0; w < DEC_WAVES; ++w) sum += acc_lds[((long)w * G + g) * dv + dim];
+    partial_o[((token * Hq + kvh * G + g) * splits + split) * dv + dim] = sum;
   }
   if (tid < G) {
     float* ml = partial_ml + ((token * Hq + kvh * G + tid) * splits + split) * 2;
@@ -989,11 +1007,12 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
   }
 }
 
-// out[token, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits that hold keys.
+// out[token, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits that hold keys
+// (dh: the width of a head's output); sigmoid: the plain sum of the splits' outputs.
 __global__ void decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
                                     const int* __restrict__ positions, int window, int page_size,
                                     int split_keys, int splits, int Hq, int dh, bf16_t* __restrict__ out,
-                                    long out_ld) {
+                                    long out_ld, int sigmoid) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int pos = positions[token];
@@ -1003,6 +1022,14 @@ __global__ void decode_merge_kernel(const float* __restrict__ partial_o, const f
   const int used = min(splits, (pos - first_page_key) / split_keys + 1);
   const float* ml = partial_ml + (token * Hq + head) * splits * 2;
   const float* o = partial_o + (token * Hq + head) * (long)splits * dh;
+  if (sigmoid) {
+    for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+      float sum = 0.f;
+      for (int s = 0; s < used; ++s) sum += o[(long)s * dh + dim];
+      out[token * out_ld + (long)head * dh + dim] = (bf16_t)sum;
+    }
+    return;
+  }
   float maximum = -INFINITY;
   for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
   float denominator = 0.f;
@@ -1018,33 +1045,40 @@ template <int DH, int G>
 static int launch_decode(const bf16_t* q, long q_ld, int T, int Hq, int Hkv, const bf16_t* k_base,
                          const bf16_t* v_base, long page_stride, int page_size, const int* block_tables,
                          int max_pages, const int* lane_of_token, const int* positions, float scale, int window,
-                         int split_keys, int splits, float* partial_o, float* partial_ml, hipStream_t stream) {
+                         int split_keys, int splits, float* partial_o, float* partial_ml, int dv,
+                         const float* head_scales, const float* score_bias, int sigmoid, hipStream_t stream) {
   const dim3 grid(splits, Hkv, T);
-  decode_attention_kernel<DH, G><<<grid, DEC_THREADS, 0, stream>>>(
+  const size_t dynamic = sizeof(float) * DEC_WAVES * G * (size_t)dv;
+  decode_attention_kernel<DH, G><<<grid, DEC_THREADS, dynamic, stream>>>(
       q, q_ld, Hq, k_base, v_base, page_stride, page_size, block_tables, max_pages, lane_of_token, positions,
-      scale, window, split_keys, splits, partial_o, partial_ml);
+      scale, window, split_keys, splits, partial_o, partial_ml, dv, head_scales, score_bias, sigmoid);
   return 0;
 }
 
 // Returns ERR_UNSUPPORTED_SIZE for shapes this kernel does not cover (the caller then uses
 // mi_paged_attention): head_dim 64 or 128, 1..8 query heads per kv head, page_size a multiple of 8,
-// split_keys a multiple of page_size and at most DEC_MAX_SPLIT.
-extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int Hkv, int dh, const void* k_base,
-                                   const void* v_base, long page_stride, int page_size, const int* block_tables,
-                                   int max_pages, const int* lane_of_token, const int* positions, float scale,
-                                   int window, int split_keys, int splits, float* partial_o, float* partial_ml,
-                                   void* out, long out_ld, hipStream_t stream) {
-  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || splits <= 0 || max_pages <= 0)
+// split_keys a multiple of page_size and at most DEC_MAX_SPLIT, values of up to 256 dims a head.
+// partial_o holds T * Hq * splits * dv floats.
+extern "C" int mi_decode_attention_forms(const void* q, long q_ld, int T, int Hq, int Hkv, int dh, int dv,
+                                         const void* k_base, const void* v_base, long page_stride, int page_size,
+                                         const int* block_tables, int max_pages, const int* lane_of_token,
+                                         const int* positions, float scale, int window, int split_keys, int splits,
+                                         float* partial_o, float* partial_ml, void* out, long out_ld,
+                                         const float* head_scales, const float* score_bias, int sigmoid,
+                                         hipStream_t stream) {
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || splits <= 0 || max_pages <= 0 || dv <= 0)
     return ERR_BAD_ARGUMENT;
   const int G = Hq / Hkv;
   if ((dh != 64 && dh != 128) || G > 8 || page_size % 8 != 0 || split_keys % page_size != 0 ||
-      split_keys <= 0 || split_keys > DEC_MAX_SPLIT || T > 65535 || Hkv > 65535)
+      split_keys <= 0 || split_keys > DEC_MAX_SPLIT || T > 65535 || Hkv > 65535 || dv > 256)
     return ERR_UNSUPPORTED_SIZE;
+  if (score_bias != nullptr && !sigmoid) return ERR_BAD_ARGUMENT;
 #define DECODE_CASE(DH_, G_)                                                                                     \
   if (dh == DH_ && G == G_)                                                                                      \
     launch_decode<DH_, G_>((const bf16_t*)q, q_ld, T, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base,     \
                            page_stride, page_size, block_tables, max_pages, lane_of_token, positions, scale,     \
-                           window, split_keys, splits, partial_o, partial_ml, stream);
+                           window, split_keys, splits, partial_o, partial_ml, dv, head_scales, score_bias,       \
+                           sigmoid, stream);
   DECODE_CASE(64, 1) DECODE_CASE(64, 2) DECODE_CASE(64, 3) DECODE_CASE(64, 4) DECODE_CASE(64, 5)
   DECODE_CASE(64, 6) DECODE_CASE(64, 7) DECODE_CASE(64, 8)
   DECODE_CASE(128, 1) DECODE_CASE(128, 2) DECODE_CASE(128, 3) DECODE_CASE(128, 4) DECODE_CASE(128, 5)
@@ -1052,10 +1086,23 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
 #undef DECODE_CASE
   RETURN_IF_LAUNCH_FAILED();
   const dim3 merge_grid(T, Hq);
-  decode_merge_kernel<<<merge_grid, dh, 0, stream>>>(partial_o, partial_ml, positions, window, page_size,
-                                                     split_keys, splits, Hq, dh, (bf16_t*)out, out_ld);
+  const int merge_threads = dv <= 64 ? 64 : dv <= 128 ? 128 : 256;
+  decode_merge_kernel<<<merge_grid, merge_threads, 0, stream>>>(partial_o, partial_ml, positions, window, page_size,
+                                                                split_keys, splits, Hq, dv, (bf16_t*)out, out_ld,
+                                                                sigmoid);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
+}
+
+// The ordinary form: softmax weights, values as wide as the keys.
+extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int Hkv, int dh, const void* k_base,
+                                   const void* v_base, long page_stride, int page_size, const int* block_tables,
+                                   int max_pages, const int* lane_of_token, const int* positions, float scale,
+                                   int window, int split_keys, int splits, float* partial_o, float* partial_ml,
+                                   void* out, long out_ld, hipStream_t stream) {
+  return mi_decode_attention_forms(q, q_ld, T, Hq, Hkv, dh, dh, k_base, v_base, page_stride, page_size, block_tables,
+                                   max_pages, lane_of_token, positions, scale, window, split_keys, splits, partial_o,
+                                   partial_ml, out, out_ld, nullptr, nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------- decode attention without a workspace argument

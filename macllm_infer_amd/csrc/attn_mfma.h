@@ -206,8 +206,9 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float p = score[t][i] == -INFINITY ? 0.f
-                                                     : 1.f / (1.f + __builtin_amdgcn_exp2f(fmaf(score[t][i], slope, offset)));
+            // the hardware's reciprocal (one unit in the last place; the weight is rounded to bfloat16 next)
+            const float weight = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(fmaf(score[t][i], slope, offset)));
+            const float p = (MASKED && score[t][i] == -INFINITY) ? 0.f : weight;
             p_frag[4 * t + i] = (bf16_t)p;
           }
 #pragma unroll

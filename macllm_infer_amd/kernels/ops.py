@@ -109,6 +109,9 @@ _SIGNATURES = {
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_long, _c_ptr],
+        "mi_decode_attention_forms": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
+                                      _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr,
+                                      _c_ptr, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_ptr],
     },
     "mamba2": {
         "mi_conv1d_silu": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -1165,45 +1168,54 @@ def prefill_attention_forms(q: torch.Tensor, num_heads: int, num_kv_heads: int, 
         _p(head_scales), _p(score_bias), _stream()), "prefill_attention_forms")
 
 
-def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:
+def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                               value_dim: Optional[int] = None) -> bool:
     """Whether the split-context kernel for single-token queries covers this geometry."""
     return (dtype == torch.bfloat16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 8
-            and page_size % 8 == 0 and page_size <= 512)
+            and page_size % 8 == 0 and page_size <= 512 and (value_dim is None or 0 < value_dim <= 256))
 
 
 def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, block_tables: torch.Tensor, lane_of_token: torch.Tensor,
                      positions: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
-                     out: torch.Tensor) -> None:
+                     out: torch.Tensor, value_dim: Optional[int] = None, head_scales: Optional[torch.Tensor] = None,
+                     score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False) -> None:
     """``paged_attention`` for batches of single decoded tokens in bfloat16: the context of each
     request is split over many workgroups and the G query heads of a kv head share its K/V
-    loads.  ``max_seq_len``: an upper bound of the longest context in the batch."""
+    loads.  ``max_seq_len``: an upper bound of the longest context in the batch.  ``value_dim``,
+    ``head_scales``, ``score_bias`` and ``sigmoid`` as in ``paged_attention``."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
+    value_dim = head_dim if value_dim is None else int(value_dim)
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "decode_attention: bfloat16 only")
-    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * head_dim) and q_ld % 8 == 0
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * value_dim) and q_ld % 8 == 0
           and q.data_ptr() % 16 == 0, "decode_attention: q/out shapes or alignment do not fit")
-    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
-    _need(decode_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size),
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype, value_dim)
+    _need(decode_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim),
           "decode_attention: geometry not covered; use paged_attention")
     _i32(block_tables, "block_tables")
     _i32(lane_of_token, "lane_of_token")
     _i32(positions, "positions")
     _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
           "decode_attention: metadata shapes do not match")
+    for name, one in (("head_scales", head_scales), ("score_bias", score_bias)):
+        _need(one is None or (one.dtype == torch.float32 and one.numel() == num_heads and one.is_contiguous()
+                              and one.is_cuda), f"decode_attention: {name} must be float32 [Hq] on the GPU")
+    _need(sigmoid or score_bias is None, "decode_attention: a bias per head is for sigmoid weights")
     span = max_seq_len if not window else min(max_seq_len, window + page_size)
     split_keys = 64
     while split_keys < 512 and span * T * num_kv_heads > 1024 * split_keys:
         split_keys *= 2
     split_keys = max(split_keys, page_size)
     splits = max(1, -(-span // split_keys))
-    partial_o = torch.empty((T, num_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+    partial_o = torch.empty((T, num_heads, splits, value_dim), dtype=torch.float32, device=q.device)
     partial_ml = torch.empty((T, num_heads, splits, 2), dtype=torch.float32, device=q.device)
-    _check(_fn("attention", "mi_decode_attention")(
-        _p(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
+    _check(_fn("attention", "mi_decode_attention_forms")(
+        _p(q), q_ld, T, num_heads, num_kv_heads, head_dim, value_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
         _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale), int(window or 0),
-        split_keys, splits, _p(partial_o), _p(partial_ml), _p(out), out_ld, _stream()), "decode_attention")
+        split_keys, splits, _p(partial_o), _p(partial_ml), _p(out), out_ld, _p(head_scales), _p(score_bias),
+        1 if sigmoid else 0, _stream()), "decode_attention")
 
 
 # --------------------------------------------------------------------------- mamba2

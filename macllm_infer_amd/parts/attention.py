@@ -225,9 +225,12 @@ class Attention(Mixer):
         plain = not sigmoid and self.head_scales is None and spec.value_width == spec.head_dim
         aligned = (qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 and out.stride(0) % 4 == 0
                    and out.data_ptr() % 8 == 0)
-        if plain and step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
+        if (step.max_query_len == 1 and aligned
+                and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2], spec.value_width)):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
-                                 step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len, out)
+                                 step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len, out,
+                                 value_dim=spec.value_width, head_scales=self.head_scales, score_bias=self.score_bias,
+                                 sigmoid=sigmoid)
         elif (plain and tiles and aligned and step.query_tile == self.query_tile
                 and ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2])):
             ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],

@@ -225,11 +225,12 @@ def test_the_projection_norm_runs_over_all_heads_at_once():
                                                  (False, 2, 1, 128, 160), (False, 4, 4, 64, 32)])
 def test_prompt_portions_in_bfloat16_run_on_the_matrix_cores(monkeypatch, sigmoid, H, G, D, V):
     """Heads of 64 and 128 in bfloat16: portions of prompts (alone and beside single tokens) go through the
-    matrix-core kernel's forms for sigmoid weights and for values of another width than the keys, single tokens
-    through the general kernel; both against the plain model, and each is seen to have run."""
+    matrix-core kernel's forms for sigmoid weights and for values of another width than the keys, steps of single
+    tokens through the kernel that splits a context over workgroups (several splits here); both against the plain
+    model, and each is seen to have run."""
     from macllm_infer_amd.kernels import ops
-    calls = {"forms": 0, "general": 0}
-    forms, general = ops.prefill_attention_forms, ops.paged_attention
+    calls = {"forms": 0, "general": 0, "decode": 0}
+    forms, general, decode = ops.prefill_attention_forms, ops.paged_attention, ops.decode_attention
 
     def spy_forms(*args, **more):
         calls["forms"] += 1
@@ -238,7 +239,12 @@ def test_prompt_portions_in_bfloat16_run_on_the_matrix_cores(monkeypatch, sigmoi
     def spy_general(*args, **more):
         calls["general"] += 1
         return general(*args, **more)
+
+    def spy_decode(*args, **more):
+        calls["decode"] += 1
+        return decode(*args, **more)
     monkeypatch.setattr(ops, "prefill_attention_forms", spy_forms)
+    monkeypatch.setattr(ops, "decode_attention", spy_decode)
     monkeypatch.setattr(ops, "paged_attention", spy_general)
     hidden, dtype = 64, torch.bfloat16
     rotation = motolix_configs.rot(2000.0, D // 2)
@@ -255,11 +261,16 @@ def test_prompt_portions_in_bfloat16_run_on_the_matrix_cores(monkeypatch, sigmoi
         spec = softmax_spec(H, G, D, V, mixer["scale"], rotation)
     harness = PartHarness(spec, tensors, hidden, dtype, page_size=16)
     first, = harness.run([("r", x[:70])])
-    second, _ = harness.run([("r", x[70:199]), ("other", x[:1])])
-    assert calls == {"forms": 2, "general": 0}
-    last, = harness.run([("r", x[199:])])
-    assert calls == {"forms": 2, "general": 1}
-    close(torch.cat([first, second, last]), want, dtype, "portions on the matrix cores")
+    second, _ = harness.run([("r", x[70:170]), ("other", x[:1])])
+    assert calls == {"forms": 2, "general": 0, "decode": 0}
+    rows = [first, second]
+    for position in range(170, 200):
+        if position % 2:
+            rows.append(harness.run([("r", x[position:position + 1])])[0])
+        else:
+            rows.append(harness.run([("other", x[position - 169:position - 168]), ("r", x[position:position + 1])])[1])
+    assert calls == {"forms": 2, "general": 0, "decode": 30}
+    close(torch.cat(rows), want, dtype, "portions on the matrix cores, single tokens over split contexts")
 
 
 def crafted_softmax(distance, length, V=8):
