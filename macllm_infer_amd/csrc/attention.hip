@@ -825,6 +825,7 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
 #define DEC_THREADS 256
 #define DEC_WAVES (DEC_THREADS / WAVE)
 #define DEC_MAX_SPLIT 512
+#define DEC_MERGE_SPLITS 256     // splits whose factors the merge keeps in LDS
 
 struct alignas(16) bf16x8 {
   bf16_t v[8];
@@ -1027,6 +1028,33 @@ __global__ void decode_merge_kernel(const float* __restrict__ partial_o, const f
       float sum = 0.f;
       for (int s = 0; s < used; ++s) sum += o[(long)s * dh + dim];
       out[token * out_ld + (long)head * dh + dim] = (bf16_t)sum;
+    }
+    return;
+  }
+  // the splits' factors exp(m_s - M) and the denominator, by the first wave (a split a lane at a time), through LDS
+  // for all; more splits than the table holds: every thread forms them for itself
+  __shared__ float factor_lds[DEC_MERGE_SPLITS];
+  __shared__ float denominator_lds;
+  if (used <= DEC_MERGE_SPLITS) {
+    if (threadIdx.x < WAVE) {
+      float maximum = -INFINITY;
+      for (int s = threadIdx.x; s < used; s += WAVE) maximum = fmaxf(maximum, ml[2 * s]);
+      maximum = wave_max(maximum);
+      float denominator = 0.f;
+      for (int s = threadIdx.x; s < used; s += WAVE) {
+        const float factor = __expf(ml[2 * s] - maximum);
+        factor_lds[s] = factor;
+        denominator += factor * ml[2 * s + 1];
+      }
+      denominator = wave_sum(denominator);
+      if (threadIdx.x == 0) denominator_lds = denominator;
+    }
+    __syncthreads();
+    const float denominator = denominator_lds;
+    for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+      float sum = 0.f;
+      for (int s = 0; s < used; ++s) sum = fmaf(factor_lds[s], o[(long)s * dh + dim], sum);
+      out[token * out_ld + (long)head * dh + dim] = (bf16_t)(sum / denominator);
     }
     return;
   }

@@ -711,6 +711,95 @@ add_layernorm_kernel(float* __restrict__ h, NormBranch b0, NormBranch b1, NormBr
     o[i] = from_float<TO>((wide_row[i] - mean) / denominator * weight[i] + bias[i]);
 }
 
+// The same for steps of few rows, whose time is the chain of waits: a thread keeps PER elements of the row in
+// registers (element threadIdx.x + k * blockDim.x), and everything the later stages read from memory (the stream's
+// row, the norms' weights and biases) is asked for at the start, beside the branches' rows.
+template <typename TO, int PER>
+__global__ void __launch_bounds__(1024)
+add_layernorm_rows_kernel(float* __restrict__ h, NormBranch b0, NormBranch b1, NormBranch b2,
+                          const float* __restrict__ vector, const float* __restrict__ weight,
+                          const float* __restrict__ bias, float eps, const float* __restrict__ branch_weight,
+                          const float* __restrict__ branch_bias, float branch_eps, TO* __restrict__ out,
+                          const int* __restrict__ rows, int d) {
+  __shared__ float scratch[16];
+  const long out_row = blockIdx.x;
+  const long row = rows ? (long)rows[out_row] : out_row;
+  float branches[PER], stream[PER], bw[PER], bb[PER], w[PER], b[PER], v[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    const bool live = i < d;
+    const long at = row * d + i;
+    branches[k] = 0.f;
+    if (live) {
+      branches[k] = branch_value(b0, at);
+      branches[k] += branch_value(b1, at);
+      branches[k] += branch_value(b2, at);
+    }
+    stream[k] = live ? h[at] : 0.f;
+    bw[k] = (live && branch_weight) ? branch_weight[i] : 0.f;
+    bb[k] = (live && branch_weight) ? branch_bias[i] : 0.f;
+    w[k] = (live && out) ? weight[i] : 0.f;
+    b[k] = (live && out) ? bias[i] : 0.f;
+    v[k] = (live && vector) ? vector[i] : 0.f;
+  }
+  if (branch_weight) {
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) sum += branches[k];
+    const float branch_mean = block_sum(sum, scratch) / (float)d;
+    float squares = 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const float centred = (int)(threadIdx.x + k * blockDim.x) < d ? branches[k] - branch_mean : 0.f;
+      squares += centred * centred;
+    }
+    const float branch_denominator = sqrtf(block_sum(squares, scratch) / (float)d + branch_eps);
+#pragma unroll
+    for (int k = 0; k < PER; ++k) v[k] += stream[k] + ((branches[k] - branch_mean) / branch_denominator * bw[k] + bb[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) v[k] += stream[k] + branches[k];
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i >= d) v[k] = 0.f;
+    else if (!rows) h[row * d + i] = v[k];
+    sum += v[k];
+  }
+  if (!out) return;
+  const float mean = block_sum(sum, scratch) / (float)d;
+  float squares = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const float centred = (int)(threadIdx.x + k * blockDim.x) < d ? v[k] - mean : 0.f;
+    squares += centred * centred;
+  }
+  const float denominator = sqrtf(block_sum(squares, scratch) / (float)d + eps);
+  TO* o = out + out_row * d;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i < d) o[i] = from_float<TO>((v[k] - mean) / denominator * w[k] + b[k]);
+  }
+}
+
+template <typename TO>
+static void launch_add_layernorm_rows(int per, int n_rows, int threads, hipStream_t stream, float* h, NormBranch b0,
+                                      NormBranch b1, NormBranch b2, const float* vector, const float* weight,
+                                      const float* bias, float eps, const float* branch_weight,
+                                      const float* branch_bias, float branch_eps, TO* out, const int* rows, int d) {
+#define ROWS_CASE(PER_)                                                                                          \
+  if (per == PER_)                                                                                               \
+    add_layernorm_rows_kernel<TO, PER_><<<n_rows, threads, 0, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, \
+                                                                        branch_weight, branch_bias, branch_eps,  \
+                                                                        out, rows, d);
+  ROWS_CASE(1) ROWS_CASE(2) ROWS_CASE(4) ROWS_CASE(8)
+#undef ROWS_CASE
+}
+
 extern "C" int mi_add_layernorm(float* h, const void* rows0, int dtype0, float factor0, const void* rows1, int dtype1,
                                 float factor1, const void* rows2, int dtype2, float factor2, const float* vector,
                                 const float* weight, const float* bias, float eps, const float* branch_weight,
@@ -721,6 +810,19 @@ extern "C" int mi_add_layernorm(float* h, const void* rows0, int dtype0, float f
   if (branch_weight && (!branch_bias || rows || !rows0)) return ERR_BAD_ARGUMENT;
   if ((size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   const NormBranch b0 = {rows0, dtype0, factor0}, b1 = {rows1, dtype1, factor1}, b2 = {rows2, dtype2, factor2};
+  if (n_rows <= 256 && d <= 8192 && (out_dtype == DT_F32 || out_dtype == DT_BF16)) {
+    // few rows: the kernel that keeps a row in registers, as many threads as a row has elements where that fits
+    const int per = d <= 1024 ? 1 : d <= 2048 ? 2 : d <= 4096 ? 4 : 8;
+    const int row_threads = (((d + per - 1) / per + WAVE - 1) / WAVE) * WAVE;
+    if (out_dtype == DT_F32)
+      launch_add_layernorm_rows<float>(per, n_rows, row_threads, stream, h, b0, b1, b2, vector, weight, bias, eps,
+                                       branch_weight, branch_bias, branch_eps, (float*)out, rows, d);
+    else
+      launch_add_layernorm_rows<bf16_t>(per, n_rows, row_threads, stream, h, b0, b1, b2, vector, weight, bias, eps,
+                                        branch_weight, branch_bias, branch_eps, (bf16_t*)out, rows, d);
+    RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   const int threads = (d > 2048 && n_rows <= 512) ? 1024 : 256;
   const size_t lds = (size_t)d * sizeof(float);
   if (out_dtype == DT_F32)

@@ -96,7 +96,18 @@ struct FusedGemmParams {
   int ssq_ld;
   // the step's rows dealt out to row_tiles workgroups per tile of features (1: every workgroup takes them all)
   int row_tiles;
+  // SWIGLU epilogue: what the gate goes through, 0 SiLU, 1 the tanh form of GELU
+  int gate_act;
 };
+
+// the gate's activation of the SWIGLU epilogue; GELU through the hardware's exponential, tanh(y) = 1 - 2 / (1 + e^(2y))
+__device__ __forceinline__ float gate_act_f(int kind, float z) {
+  if (kind == 1) {
+    const float y = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+    return z * (1.0f - __frcp_rn(1.0f + __expf(2.0f * y)));
+  }
+  return silu_f(z);
+}
 
 // What is left of a step for a workgroup that takes `rows` of its rows from row0 on (plain prologue).
 __device__ __forceinline__ void take_rows(FusedGemmParams& p, int row0, int rows) {
@@ -586,7 +597,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         if (m >= p.M || column >= half_rows) continue;
         const float gate = round_bf16(tile[i * (MT * 16) + m]);
         const float up = round_bf16(tile[(8 + i) * (MT * 16) + m]);
-        reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + column] = (bf16_t)(silu_f(gate) * up);
+        reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + column] = (bf16_t)(gate_act_f(p.gate_act, gate) * up);
       }
     }
   }
@@ -897,7 +908,7 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
         if (tile0 + nt >= tiles || q >= 2 || m >= p.M) continue;
         bf16x4_t packed;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(silu_f(round_bf16(v[i])) * round_bf16(up[i]));
+        for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(gate_act_f(p.gate_act, round_bf16(v[i])) * round_bf16(up[i]));
         bf16_t* to = out + (long)m * p.out_ld + column;
         if (p.out_ld % 4 == 0) {
           *reinterpret_cast<bf16x4_t*>(to) = packed;
@@ -979,6 +990,10 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                              int feature_tiles, int w_fragments, const float* ssq_in, int ssq_blocks, int ssq_width,
                              float ssq_eps, int row_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
+  // the bits of epi above the lowest eight: the gate's activation of the SWIGLU epilogue (0 SiLU, 1 GELU, tanh form)
+  const int gate_act = epi >> 8;
+  epi &= 0xff;
+  if (gate_act < 0 || gate_act > 1 || (gate_act && epi != EPI_SWIGLU)) return ERR_BAD_ARGUMENT;
   if (ssq_in && (pro != PRO_PLAIN || ssq_blocks <= 0 || ssq_width <= 0)) return ERR_BAD_ARGUMENT;
   const bool shared_rows = feature_tiles < 0;       // -1, -2: that many tiles a wave of shared_rows_gemm_kernel
   if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || out_f32)) return ERR_BAD_ARGUMENT;
@@ -997,6 +1012,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   if (pro != PRO_NORM && pro != PRO_PLAIN) return ERR_BAD_ARGUMENT;
   if (!shared_rows && fused_gemm_lds(MT, pro, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
+  p.gate_act = gate_act;
   p.h_in = h_in;
   p.delta0 = (const bf16_t*)delta0;
   p.delta1 = (const bf16_t*)delta1;

@@ -1549,13 +1549,15 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
                deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
                conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None,
-               row_scale: Optional["RowScale"] = None, shared_rows: bool = False, row_tiles: int = 1) -> None:
+               row_scale: Optional["RowScale"] = None, shared_rows: bool = False, row_tiles: int = 1,
+               gate_activation: str = "silu") -> None:
     """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
 
     Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
     the rows are summed (the sum goes to ``h_out``, a different tensor, if given), RMS-normed
     with ``norm_weight`` and ``eps``.  Epilogue PLAIN: bfloat16 or float32 ``out`` [M, N] times
-    ``out_scale``.  SWIGLU: weight rows in tiles of 8 gate + 8 up rows, ``out`` [M, N/2].
+    ``out_scale``.  SWIGLU: weight rows in tiles of 8 gate + 8 up rows, ``out`` [M, N/2] = act(gate) * up with
+    act = SiLU or, ``gate_activation`` "gelu_tanh", the tanh form of GELU.
     CONV: ``conv`` = {lo, hi, taps, weight [C, taps], bias, state [slots, taps-1, C], slot_ids}:
     rows lo..hi-1 go through the causal depthwise conv step of their channel with the request's
     tail (which is rolled) and SiLU.  ``feature_tiles`` (1, 2 or 4; more than one with ``x`` only): how many
@@ -1571,6 +1573,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
     _need(row_scale is None or x is not None, "fused_gemm: a row scale needs x")
+    _need(gate_activation in GATE_ACTIVATIONS and (gate_activation == "silu" or epilogue == EPI_SWIGLU),
+          "fused_gemm: the gate's activation is silu or gelu_tanh, and belongs to the SWIGLU epilogue")
     _need(1 <= row_tiles <= 4 and (row_tiles == 1 or (x is not None and feature_tiles == 1 and not shared_rows)),
           "fused_gemm: row_tiles is 1 to 4, and more than 1 needs x, one feature tile and the skinny kernel")
     if row_scale is not None:
@@ -1616,7 +1620,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _i32(slot_ids, "slot_ids")
         _need(slot_ids.numel() >= M, "fused_gemm: one slot per row")
     _check(_fn("decode", "mi_fused_gemm")(
-        pro, epilogue, _p(h_in), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
+        pro, epilogue | (GATE_ACTIVATIONS[gate_activation] << 8), _p(h_in), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
         _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm")),
         _p(bias), M, N, K, _p(out), out_ld,
         1 if out.dtype == torch.float32 else 0, float(out_scale), lo, hi, taps, _p(conv_w), _p(conv_b), _p(conv_state),

@@ -54,6 +54,17 @@ class SwiGLU(FeedForward):
         return self.gate_up, self.down, self.tile
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rows, width = x.shape
+        if (self.tile == 8 and x.dtype == torch.bfloat16 and self.gate_up.weight.dtype == torch.bfloat16
+                and rows <= ops.SKINNY_ROWS and width % 32 == 0
+                and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                and ops.fused_gemm_supported(False, rows, width)):
+            # a step of a few rows: the gate's activation and the product with the up half in the skinny kernel's
+            # epilogue (the weight rows already lie in its tiles of 8 gate and 8 up rows)
+            activated = torch.empty((rows, self.spec.intermediate_size), dtype=x.dtype, device=x.device)
+            ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, x=x, epilogue=ops.EPI_SWIGLU,
+                           gate_activation=self.spec.activation)
+            return self.down(activated)
         gate_up = self.gate_up(x)
         activated = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=gate_up.dtype, device=x.device)
         ops.swiglu(gate_up, activated, self.tile, activation=self.spec.activation)
