@@ -198,7 +198,7 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
             out[token, head * value_dim:(head + 1) * value_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
 
 
-def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size):
+def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim=None):
     return False
 
 
@@ -207,9 +207,10 @@ def prefill_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_s
 
 
 def decode_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
-                     scale, window, max_seq_len, out):
+                     scale, window, max_seq_len, out, value_dim=None, head_scales=None, score_bias=None, sigmoid=False):
     paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
-                    scale, window, out)
+                    scale, window, out, value_dim=value_dim, head_scales=head_scales, score_bias=score_bias,
+                    sigmoid=sigmoid)
 
 
 def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out):
