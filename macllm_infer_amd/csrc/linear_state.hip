@@ -36,6 +36,7 @@
 //   scan    every chunk from its starting state: the outputs, and behind a lane's last chunk the state of the request.
 // All of it in float32: the passes add the same products in another order.
 #include "common.h"
+#include <cstdint>
 
 #define LS_MAX_PER_LANE 16          // key channels of a column that one lane keeps
 #define LS_THREADS 256
@@ -69,6 +70,7 @@ struct ScanArgs {
   const int* lane_chunks;           // [lanes, 2] = (first chunk, chunks)
   float* local;                     // [chunks, H, dv (+ dk), dk]: what the local pass leaves
   float* start;                     // [chunks, H, dv, dk]: every chunk's starting state
+  int whole_fours;                  // dk a multiple of 4 and the state tables 16-byte aligned: states move 4 floats a load
 };
 
 #define LS_RETENTION 0              // the kinds of recurrence
@@ -159,6 +161,7 @@ linear_state_scan_kernel(const ScanArgs a) {
 
   // the columns' share of the state
   float s[CPL][PL];
+  const bool whole_fours = a.whole_fours != 0;
   const long state_head = ((long)a.slot_ids[lane_of_step] * a.H + head) * dv;
 #pragma unroll
   for (int c = 0; c < CPL; ++c) {
@@ -166,6 +169,20 @@ linear_state_scan_kernel(const ScanArgs a) {
     const bool mine = in_group && column_in_group + c < a.columns && column < total_columns;
     const float* from = a.state + (state_head + (mine && column < dv ? column : 0)) * dk;
     if (MODE == LS_CHUNK) from = a.start + (((long)blockIdx.x * a.H + head) * dv + (mine ? column : 0)) * dk;
+    if (MODE != LS_LOCAL && whole_fours) {
+      // dk a multiple of 4: a lane's run of channels is whole groups of four, 16 bytes a load
+#pragma unroll
+      for (int g = 0; g < PL / 4; ++g) {
+        const int channel = channel0 + 4 * g;
+        const bool held = mine && 4 * g < per_lane && channel < dk;
+        const float4 four = held ? *reinterpret_cast<const float4*>(from + channel) : make_float4(0.f, 0.f, 0.f, 0.f);
+        s[c][4 * g + 0] = four.x;
+        s[c][4 * g + 1] = four.y;
+        s[c][4 * g + 2] = four.z;
+        s[c][4 * g + 3] = four.w;
+      }
+      continue;
+    }
 #pragma unroll
     for (int e = 0; e < PL; ++e) {
       const int channel = channel0 + e;
@@ -352,10 +369,20 @@ linear_state_scan_kernel(const ScanArgs a) {
     float* into = a.state + (state_head + (mine && column < dv ? column : 0)) * dk;
     if (MODE == LS_LOCAL) into = a.local + (((long)blockIdx.x * a.H + head) * total_columns + (mine ? column : 0)) * dk;
     if (mine && (MODE != LS_CHUNK || last_of_lane)) {
+      if (whole_fours) {
 #pragma unroll
-      for (int e = 0; e < PL; ++e) {
-        const int channel = channel0 + e;
-        if (e < per_lane && channel < dk) into[channel] = s[c][e];
+        for (int g = 0; g < PL / 4; ++g) {
+          const int channel = channel0 + 4 * g;
+          if (4 * g < per_lane && channel < dk)
+            *reinterpret_cast<float4*>(into + channel) =
+                make_float4(s[c][4 * g + 0], s[c][4 * g + 1], s[c][4 * g + 2], s[c][4 * g + 3]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < PL; ++e) {
+          const int channel = channel0 + e;
+          if (e < per_lane && channel < dk) into[channel] = s[c][e];
+        }
       }
     }
   }
@@ -470,6 +497,7 @@ static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, 
   a.logits_ld = logits_ld; a.decay_bias = decay_bias; a.decay_floor = decay_floor; a.key_eps = key_eps;
   a.gate_power = gate_power; a.query_scale = query_scale;
   a.chunks = nullptr; a.lane_chunks = nullptr; a.local = nullptr; a.start = nullptr;
+  a.whole_fours = (dk % 4 == 0 && (uintptr_t)state % 16 == 0) ? 1 : 0;
   int R = 1;
   while (R * LS_MAX_PER_LANE < dk) R *= 2;
   a.R = R;
@@ -579,6 +607,7 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
                        decay_bias, decay_floor, key_eps, gate_power, query_scale);
   if (code) return code;
   a.chunks = chunks; a.lane_chunks = lane_chunks; a.local = local; a.start = start;
+  if ((uintptr_t)local % 16 != 0 || (uintptr_t)start % 16 != 0) a.whole_fours = 0;
   const int kind = removal_col >= 0 ? LS_DELTA : gate_power > 0.f ? LS_GATED : LS_RETENTION;
   size_t lds;
   int splits;
