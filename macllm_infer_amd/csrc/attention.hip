@@ -142,6 +142,25 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
   float* q_lds = prepared_row;
   float* k_lds = q_lds + q_cols;
   float* v_lds = k_lds + k_cols;
+  // the token's turns, (cosine, sine) a pair of dims, once for all heads: keys' pairs, then the values'
+  const int half = rotary_dim / 2;
+  const int value_half = dv / 2;
+  float* turns = v_lds + v_cols;
+  float* value_turns = turns + 2 * half;
+  if (inv_freq)
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      float sine, cosine;
+      sincosf(position * inv_freq[j], &sine, &cosine);
+      turns[2 * j] = cosine;
+      turns[2 * j + 1] = sine;
+    }
+  if (value_inv_freq)
+    for (int m = threadIdx.x; m < value_half; m += blockDim.x) {
+      float sine, cosine;
+      sincosf(position * value_inv_freq[m], &sine, &cosine);
+      value_turns[2 * m] = cosine;
+      value_turns[2 * m + 1] = sine;
+    }
   float q_squares = 0.f, k_squares = 0.f;
   for (int i = threadIdx.x; i < q_cols + k_cols; i += blockDim.x) {
     const float x = to_float(row[i]);
@@ -166,7 +185,6 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
     offset = (int)(cell - page * page_size);
   }
   // q heads then k heads: a thread an element; the partner of a turned element is read from LDS, which nobody writes
-  const int half = rotary_dim / 2;
   for (int item = threadIdx.x; item < q_cols + k_cols; item += blockDim.x) {
     const int head = item / dh;
     const int j = item - head * dh;
@@ -174,9 +192,8 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
     float value = x[j];
     if (inv_freq && j < rotary_dim) {
       const bool low = j < half;
-      const float angle = position * inv_freq[low ? j : j - half];
-      float sine, cosine;
-      sincosf(angle, &sine, &cosine);
+      const int pair = low ? j : j - half;
+      const float cosine = turns[2 * pair], sine = turns[2 * pair + 1];
       const float partner = x[low ? j + half : j - half];
       value = low ? value * cosine - partner * sine : value * cosine + partner * sine;
     }
@@ -185,16 +202,14 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
       k_base[page * page_stride + ((long)(head - Hq) * page_size + offset) * dh + j] = from_float<T>(value);
   }
   if (cell >= 0) {
-    const int value_half = dv / 2;
     for (int item = threadIdx.x; item < v_cols; item += blockDim.x) {
       const int kvh = item / dv;
       const int i = item - kvh * dv;
       float value = v_lds[item];
       if (value_inv_freq) {
         const bool low = i < value_half;
-        const float angle = position * value_inv_freq[low ? i : i - value_half];
-        float sine, cosine;
-        sincosf(angle, &sine, &cosine);
+        const int pair = low ? i : i - value_half;
+        const float cosine = value_turns[2 * pair], sine = value_turns[2 * pair + 1];
         const float partner = v_lds[kvh * dv + (low ? i + value_half : i - value_half)];
         value = low ? value * cosine - partner * sine : value * cosine + partner * sine;
       }
@@ -216,7 +231,8 @@ extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq
   if (ld < (long)(Hq + Hkv) * dh + (values_from_keys ? 0L : (long)Hkv * dv)) return ERR_BAD_ARGUMENT;
   if (slot_mapping && (!k_base || !v_base || page_size <= 0)) return ERR_BAD_ARGUMENT;
   if (!inv_freq) rotary_dim = 0;
-  const size_t lds = ((size_t)(Hq + Hkv) * dh + (size_t)Hkv * dv) * sizeof(float);
+  // the row, and (cosine, sine) of the keys' and the values' pairs
+  const size_t lds = ((size_t)(Hq + Hkv) * dh + (size_t)Hkv * dv + (size_t)rotary_dim + (size_t)(dv / 2) * 2) * sizeof(float);
   if (lds > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   if (dtype == DT_F32)
     attention_prepare_kernel<float><<<T, 256, lds, stream>>>((float*)qkv, ld, Hq, Hkv, dh, dv, values_from_keys, positions,
