@@ -428,8 +428,41 @@ def test_the_gelu_gated_feed_forward_alone(dtype, hidden, inner, T):
     close(got, want, dtype, "feed-forward")
 
 
+@pytest.mark.parametrize("hidden, inner, T", [(256, 136, 1), (64, 48, 9), (2560, 4104, 16), (96, 8, 17)])
+def test_small_steps_in_bfloat16_gate_in_the_epilogue_of_their_product(monkeypatch, hidden, inner, T):
+    """Weights stored in bfloat16 and up to 16 rows: act(gate) * up leaves the skinny product's epilogue (seen to have
+    run, with the GELU), more rows go through the separate kernel; both against the plain implementation."""
+    from macllm_infer_amd.config import SwiGLUSpec
+    from macllm_infer_amd.kernels import build, ops
+    from macllm_infer_amd.parts import BuildContext, part_class
+    calls = []
+    fused = ops.fused_gemm
+
+    def spy(*args, **more):
+        calls.append((more.get("epilogue"), more.get("gate_activation")))
+        return fused(*args, **more)
+    monkeypatch.setattr(ops, "fused_gemm", spy)
+    dtype = torch.bfloat16
+    context = BuildContext(hidden_size=hidden, dtype=dtype, device=torch.device(DEV), max_context=64)
+    build.ensure_modules(("common", "gemm", "decode"))
+    tensors = {"p.gate_proj.weight": rand(inner, hidden, seed=1, scale=2.0 * hidden ** -0.5).to(dtype),
+               "p.up_proj.weight": rand(inner, hidden, seed=2, scale=hidden ** -0.5).to(dtype),
+               "p.down_proj.weight": rand(hidden, inner, seed=3, scale=inner ** -0.5).to(dtype)}
+    spec = SwiGLUSpec(intermediate_size=inner, activation="gelu_tanh")
+    ffn = part_class(spec)(spec, "p", tensors, context)
+    x = rand(T, hidden, seed=4, scale=1.5).to(dtype)
+    got = ffn.forward(x.to(DEV)).float().cpu()
+    names = {"p.gate": tensors["p.gate_proj.weight"].double(), "p.up": tensors["p.up_proj.weight"].double(),
+             "p.down": tensors["p.down_proj.weight"].double()}
+    want = motolix_plain.feed_forward(x.double(), "p", names)
+    assert ((ops.EPI_SWIGLU, "gelu_tanh") in calls) == (T <= 16)
+    close(got, want, dtype, "feed-forward")
+
+
+# few rows keep a row in registers (one to eight elements a thread), many rows or wide ones lay it in LDS
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hidden, T, count", [(40, 19, 2), (328, 7, 1), (4104, 3, 2), (9000, 2, 1)])
+@pytest.mark.parametrize("hidden, T, count", [(40, 19, 2), (328, 7, 1), (1500, 64, 2), (4104, 3, 2), (8192, 2, 1),
+                                              (9000, 2, 1), (328, 300, 2), (2560, 257, 1)])
 def test_a_branch_joins_the_stream_through_a_norm_of_its_own(dtype, hidden, T, count):
     """x <- x + LN_b(sum of factor * branch), then LN(x): the stream stays float32, the sum of the branches is
     never rounded; with an offset in the branches that a norm without centring would keep."""
