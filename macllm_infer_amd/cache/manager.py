@@ -29,11 +29,13 @@ from .pages import BlockTable, CacheExhausted, PagePool, SlotPool
 class KVNeed:
     """Token-proportional cache: per token, keys of ``num_kv_heads`` x ``head_dim`` and values of
     ``num_kv_heads`` x ``value_dim`` (None: the keys' width); ``window`` = how many of the most recent
-    tokens must stay (None = all)."""
+    tokens must stay (None = all); ``keep_first`` = how many of a request's first tokens stay as well, however
+    far the window has moved on."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    keep_first: int = 0
     token_proportional = True             # what tells this need from one of fixed size, whatever its class
 
     @property
@@ -65,7 +67,7 @@ class Core:
     and block tables, the slot pool and the requests' lengths."""
 
     def __init__(self, page_sizes: Sequence[int], num_pages: Sequence[int], windows: Sequence[Optional[int]],
-                 max_requests: int):
+                 max_requests: int, kept_first: Optional[Sequence[int]] = None):
         self.lib = native.lib()
         sizes, pages = native.as_ints(list(page_sizes)), native.as_ints(list(num_pages))
         spans = native.as_ints([window or -1 for window in windows])
@@ -73,6 +75,9 @@ class Core:
                                           native.int_pointer(spans), max_requests)
         if not self.pointer:
             raise ValueError("page sizes, page counts and the number of requests must be positive")
+        for group, tokens in enumerate(kept_first or ()):
+            if tokens and self.lib.hc_keep_first(self.pointer, group, int(tokens)) != 0:
+                raise ValueError("the first tokens a window keeps cannot be negative")
 
     def __del__(self):
         if getattr(self, "pointer", None):
@@ -192,7 +197,8 @@ class CacheManager:
                     raise TypeError(f"unknown cache need {need!r}")
             self.entries[key] = entry
         self.core = Core([group.page_size for group in self.groups], [group.num_pages for group in self.groups],
-                         [group.need.window for group in self.groups], max_requests)
+                         [group.need.window for group in self.groups], max_requests,
+                         [getattr(group.need, "keep_first", 0) for group in self.groups])
         self.slots = SlotPool.view(self.core.lib.hc_slot_pool(self.core.pointer), self.core)
         for index, group in enumerate(self.groups):
             group.pool = PagePool.view(self.core.lib.hc_group_pool(self.core.pointer, index), self.core)

@@ -32,6 +32,7 @@ def lib() -> ctypes.CDLL:
             "hc_pool_free_count": (i, [p]), "hc_pool_take": (i, [p, i, _INT_P]),
             "hc_pool_give": (i, [p, _INT_P, i]), "hc_pool_check": (i, [p, _INT_P, i]),
             "hc_create": (p, [i, _INT_P, _INT_P, _INT_P, i]), "hc_destroy": (None, [p]),
+            "hc_keep_first": (i, [p, i, i]),
             "hc_group_pool": (p, [p, i]), "hc_slot_pool": (p, [p]), "hc_add_request": (i, [p]),
             "hc_finish": (i, [p, i]), "hc_length": (i, [p, i]), "hc_lengths": (None, [p, i, _INT_P, _INT_P]),
             "hc_reserve": (i, [p, i, _INT_P, _INT_P, _INT_P]), "hc_commit": (i, [p, i, _INT_P, _INT_P]),

@@ -42,12 +42,37 @@ class WavelengthScalingSpec:
 
 
 @dataclass(frozen=True)
+class RampScalingSpec:
+    """Frequencies blended with their ``factor``-th part by a ramp over the pair index i (YaRN): with
+    where(t) = dims * ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(where(fast)), 0),
+    hi = min(ceil(where(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, ``min_span``), 0, 1) the
+    frequency is f_i / factor * ramp_i + f_i * (1 - ramp_i); cosines and sines are multiplied by
+    ``magnitude_slope`` * ln(factor) + 1."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
+    magnitude_slope: float = 0.1
+    min_span: float = 0.001
+
+    def validate(self) -> None:
+        _require(self.factor > 0 and self.original > 0, "rope scaling needs a positive factor and original context")
+        _require(self.fast > 0 and self.slow > 0, "rope scaling needs positive numbers of turns (fast, slow)")
+
+    @property
+    def magnitude(self) -> float:
+        import math
+        return self.magnitude_slope * math.log(self.factor) + 1.0
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Half-split rotary position encoding of the first ``rotary_dim`` dims of a head
-    (src/architecture.rs:44-62).  ``scaling``: the frequencies are stretched by wavelength (None: as they are)."""
+    (src/architecture.rs:44-62).  ``scaling``: the frequencies are stretched by wavelength
+    (``WavelengthScalingSpec``) or blended by a ramp (``RampScalingSpec``); None: as they are."""
     theta: float
     rotary_dim: int
-    scaling: Optional[WavelengthScalingSpec] = None
+    scaling: Optional[object] = None
     kind: str = "rope"
 
     def validate(self, head_dim: int) -> None:
@@ -83,9 +108,10 @@ class RmsNormSpec:
 class InterleavedRopeSpec:
     """Rotary position encoding whose pairs are neighbours: dimension 2i turns with dimension 2i + 1, i below
     ``rotary_dim`` / 2, by the angle position * theta^(-2i / rotary_dim); dimensions from ``rotary_dim`` on pass
-    unchanged."""
+    unchanged.  ``scaling``: as for ``RopeSpec``."""
     theta: float
     rotary_dim: int
+    scaling: Optional[object] = None
     kind: str = "rope_interleaved"
 
     def validate(self, head_dim: int) -> None:
@@ -93,6 +119,8 @@ class InterleavedRopeSpec:
                  f"rope theta must be finite and positive, got {self.theta}")
         _require(0 < self.rotary_dim <= head_dim and self.rotary_dim % 2 == 0,
                  f"rotary_dim {self.rotary_dim} must be even and in 2..={head_dim}")
+        if self.scaling is not None:
+            self.scaling.validate()
 
 
 @dataclass(frozen=True)
@@ -155,6 +183,21 @@ class AttentionSpec:
     # value_rotation_theta^(-2m / value width)) before they are cached, and every head's output is turned back by
     # its query's position; None: values as projected
     value_rotation_theta: Optional[float] = None
+    # with a window: keys at positions below ``keep_first`` stay visible to every later query, at their true
+    # positions, however far the window has moved on
+    keep_first: int = 0
+    # a sink whose score is this fixed number (no tensor): exp(fixed_sink) is one more term of the denominator
+    fixed_sink: Optional[float] = None
+    # a causal convolution over time on every channel of the q, k and v projections, right behind the products
+    # (tensors ``q_proj.conv`` ... [channels, taps], no bias, no activation); the last taps - 1 projected rows of a
+    # request are part of its state.  0: none
+    conv_kernel: int = 0
+    # an RMS norm of every q head and every k head over ``head_dim`` (``head_norm_eps`` inside the root):
+    # "before_rotation" or "after_rotation"; with ``head_norm_weight`` times a weight of ``head_dim`` numbers that
+    # all heads share (tensors ``q_norm`` / ``k_norm``), else the bare division.  None: no such norm
+    head_norm: Optional[str] = None
+    head_norm_weight: bool = False
+    head_norm_eps: float = 1e-6
     kind: str = "attention"
 
     @property
@@ -181,6 +224,15 @@ class AttentionSpec:
         if self.value_rotation_theta is not None:
             _require(self.value_rotation_theta > 0 and self.value_width % 2 == 0,
                      "turned values need a positive base and an even width")
+        _require(self.keep_first >= 0, "the number of first tokens a window keeps cannot be negative")
+        _require(self.fixed_sink is None or (not self.sink and self.weighting == "softmax"),
+                 "a fixed sink stands in a softmax, in place of a learned one")
+        _require(0 <= self.conv_kernel, "the taps of the projections' convolution cannot be negative")
+        _require(self.head_norm in (None, "before_rotation", "after_rotation"),
+                 f"the heads' norm {self.head_norm!r} is not known")
+        _require(self.head_norm is None or self.projection_norm_eps is None,
+                 "q and k are normed head by head or as whole projections, not both")
+        _require(self.head_norm is None or self.head_norm_eps > 0, "the heads' norm eps must be positive")
         self.position.validate(self.head_dim)
 
 
@@ -188,8 +240,8 @@ class AttentionSpec:
 class LatentAttentionSpec:
     """Causal softmax attention whose queries, keys and values come through low-rank latents.
 
-    Queries: c_q = RMSNorm(W_dq h) [``q_rank``], q = W_uq c_q, per head ``head_dim`` plain dimensions followed by
-    ``rope_dim`` turned ones.  Keys and values: W_dkv h gives ``kv_rank`` + ``rope_dim`` numbers; the first
+    Queries: c_q = RMSNorm(W_dq h) [``q_rank``], q = W_uq c_q (``q_rank`` None: q = W_q h, no latent), per head
+    ``head_dim`` plain dimensions followed by ``rope_dim`` turned ones.  Keys and values: W_dkv h gives ``kv_rank`` + ``rope_dim`` numbers; the first
     ``kv_rank``, RMS-normed, are the latent c, the rest is one turned key part shared by all heads.  A head's plain
     key is W_uk c, its value W_uv c (``value_dim`` wide); score = (q_plain . k_plain + q_turned . k_turned) *
     ``scale``.  The cache holds c and the turned key part of a token, nothing per head.  ``position`` turns the
@@ -198,7 +250,7 @@ class LatentAttentionSpec:
     head_dim: int
     rope_dim: int
     value_dim: int
-    q_rank: int
+    q_rank: Optional[int]
     kv_rank: int
     scale: float
     norm_eps: float
@@ -212,8 +264,9 @@ class LatentAttentionSpec:
         return self.kv_rank + self.rope_dim
 
     def validate(self) -> None:
-        for name in ("num_heads", "head_dim", "value_dim", "q_rank", "kv_rank"):
+        for name in ("num_heads", "head_dim", "value_dim", "kv_rank"):
             _require(getattr(self, name) > 0, f"latent attention {name} must be positive")
+        _require(self.q_rank is None or self.q_rank > 0, "latent attention q_rank must be positive")
         _require(self.rope_dim >= 0, "latent attention rope_dim cannot be negative")
         _require(self.scale > 0, "attention scale must be positive")
         _require(self.norm_eps > 0, "latent attention norm eps must be positive")
@@ -235,26 +288,41 @@ class ClampedGLUSpec:
 
 
 @dataclass(frozen=True)
+class PowerReluSpec:
+    """The activation of a feed-forward without a gate: act(z) = max(z, 0)^2 (an expert is then
+    down(act(up(x))), with no gate matrix)."""
+    gated = False
+
+    def validate(self) -> None:
+        return None
+
+
+@dataclass(frozen=True)
 class RoutedExpertsSpec:
-    """A mixture of ``num_experts`` small gated feed-forwards (``expert_size`` wide, no biases) of which a token
+    """A mixture of ``num_experts`` small feed-forwards (``expert_size`` wide, no biases) of which a token
     uses ``top_k``, and optionally a shared one (``shared_size`` wide) that every token uses, times
-    sigmoid(w_sg . x).  Router: s = softmax(W_router x) over all experts in float32; the ``top_k`` largest of
-    s + correction are chosen; their weights are their s divided by the sum of the chosen s (+ ``weight_eps``),
-    times ``route_scale``."""
+    sigmoid(w_sg . x).  An expert is gated (``ClampedGLUSpec``: gate, up, down) or not (``PowerReluSpec``: up, down).
+    Router, ``routing`` "softmax_then_top": s = softmax(W_router x) over all experts in float32; the ``top_k``
+    largest of s + correction are chosen; their weights are their s divided by the sum of the chosen s
+    (+ ``weight_eps``), times ``route_scale``.  ``routing`` "top_then_softmax": the ``top_k`` largest logits
+    z = W_router x + bias (tensor ``router.bias``) are chosen and weighted by the softmax over the chosen logits
+    alone, times ``route_scale``."""
     num_experts: int
     top_k: int
     expert_size: int
-    activation: ClampedGLUSpec
+    activation: object
     route_scale: float = 1.0
     weight_eps: float = 1e-20
     shared_size: Optional[int] = None
     shared_activation: Optional[ClampedGLUSpec] = None
+    routing: str = "softmax_then_top"
     kind: str = "routed_experts"
 
     def validate(self) -> None:
         _require(self.num_experts > 0 and self.expert_size > 0, "the experts' number and width must be positive")
         _require(0 < self.top_k <= self.num_experts,
                  f"a token uses {self.top_k} experts of {self.num_experts}")
+        _require(self.routing in ("softmax_then_top", "top_then_softmax"), f"routing {self.routing!r} is not known")
         self.activation.validate()
         if self.shared_size is not None:
             _require(self.shared_size > 0 and self.shared_activation is not None,
@@ -306,7 +374,13 @@ class Mamba2Spec:
     in_multiplier: float = 1.0
     out_multiplier: float = 1.0
     multipliers: Tuple[float, float, float, float, float] = (1.0, 1.0, 1.0, 1.0, 1.0)
+    # equal parts of the gated rows that the gated norm divides by their own root mean square (None: ``num_groups``)
+    norm_groups: Optional[int] = None
     kind: str = "mamba2"
+
+    @property
+    def norm_parts(self) -> int:
+        return self.num_groups if self.norm_groups is None else self.norm_groups
 
     @property
     def inner_size(self) -> int:
@@ -328,6 +402,8 @@ class Mamba2Spec:
         _require(self.inner_size % self.num_groups == 0, "mamba inner size must divide into its groups")
         _require(len(self.multipliers) == 5, "ssm_multipliers must have 5 entries (z, x, B, C, dt)")
         _require(self.norm_eps > 0, "mamba norm eps must be positive")
+        _require(self.norm_parts > 0 and self.inner_size % self.norm_parts == 0,
+                 "mamba inner size must divide into the parts of its gated norm")
 
 
 @dataclass(frozen=True)
@@ -435,6 +511,10 @@ class MixerSlot:
     name: str
     spec: object
     weight: float = 1.0
+    # an RMS norm of the mixer's output over the model width (``RmsNormSpec``, tensor ``<name>.<post_norm_name>``)
+    # before the weighted sum of the layer's mixers; None: the output as it is
+    post_norm: object = None
+    post_norm_name: str = "out"
 
 
 @dataclass(frozen=True)
@@ -551,6 +631,8 @@ class ModelSpec:
             _require(len(set(names)) == len(names), f"layer {layer.prefix} names a mixer twice")
             for slot in layer.mixers:
                 slot.spec.validate()
+                if slot.post_norm is not None:
+                    slot.post_norm.validate()
             layer.mixer_norm.validate()
             if layer.mixer_post_norm is not None:
                 layer.mixer_post_norm.validate()

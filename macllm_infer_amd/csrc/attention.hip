@@ -120,8 +120,12 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 // float32 arithmetic on that copy:
 //   * q_norm / k_norm (optional): the whole q projection (Hq * dh numbers), and the whole k projection, is divided by
 //     its root mean square (eps inside the root) and multiplied by a weight of that length, before rotation;
-//   * q and k are turned by the token's position (half-split pairs over the first rotary_dim dims, angle =
-//     (float)position * inv_freq[j]); q is written back in place, k goes to the token's cache cell;
+//   * head_norm (1: before the rotation, 2: after it): every q head and every k head is divided by its own root mean
+//     square over dh (head_eps inside the root) and multiplied by q_head_weight / k_head_weight (float32 [dh], one
+//     weight for all heads; null: the bare division);
+//   * q and k are turned by the token's position over the first rotary_dim dims, angle = (float)position *
+//     inv_freq[j], pairs (j, j + rotary_dim / 2) or, interleaved, (2j, 2j + 1); cosines and sines times turn_scale;
+//     q is written back in place, k goes to the token's cache cell;
 //   * the values are the v heads of the row or, with values_from_keys, the k heads as they were projected (before
 //     norm and rotation; dv = dh); with value_inv_freq they are turned by the position over all dv dims (half-split
 //     pairs, angle = (float)position * value_inv_freq[m]); they go to the token's transposed cache cell.
@@ -129,7 +133,10 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, int dv, int values_from_keys,
                          const int* __restrict__ positions, const float* __restrict__ inv_freq, int rotary_dim,
+                         int interleaved, float turn_scale,
                          const float* __restrict__ q_norm, const float* __restrict__ k_norm, float norm_eps,
+                         int head_norm, const float* __restrict__ q_head_weight, const float* __restrict__ k_head_weight,
+                         float head_eps,
                          const float* __restrict__ value_inv_freq, const int* __restrict__ slot_mapping,
                          T* __restrict__ k_base, T* __restrict__ v_base, long page_stride, int page_size) {
   extern __shared__ float prepared_row[];
@@ -151,8 +158,8 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       float sine, cosine;
       sincosf(position * inv_freq[j], &sine, &cosine);
-      turns[2 * j] = cosine;
-      turns[2 * j + 1] = sine;
+      turns[2 * j] = cosine * turn_scale;
+      turns[2 * j + 1] = sine * turn_scale;
     }
   if (value_inv_freq)
     for (int m = threadIdx.x; m < value_half; m += blockDim.x) {
@@ -177,6 +184,37 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
     for (int i = threadIdx.x; i < k_cols; i += blockDim.x) k_lds[i] = k_lds[i] / k_rms * k_norm[i];
   }
   __syncthreads();
+  // a head's root mean square: one wave a head, the lanes' shares added in an order that dh alone fixes
+  auto norm_heads = [&]() {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int waves = blockDim.x / WAVE;
+    for (int head = threadIdx.x / WAVE; head < Hq + Hkv; head += waves) {
+      float* x = prepared_row + (long)head * dh;
+      const float* weight = head < Hq ? q_head_weight : k_head_weight;
+      float squares = 0.f;
+      for (int j = lane; j < dh; j += WAVE) squares = fmaf(x[j], x[j], squares);
+      const float rms = sqrtf(wave_sum(squares) / (float)dh + head_eps);
+      for (int j = lane; j < dh; j += WAVE) x[j] = weight ? x[j] / rms * weight[j] : x[j] / rms;
+    }
+    __syncthreads();
+  };
+  if (head_norm == 1) norm_heads();
+  // q heads then k heads: a thread a pair of dims, turned in place in LDS
+  if (inv_freq && half > 0) {
+    for (int item = threadIdx.x; item < (Hq + Hkv) * half; item += blockDim.x) {
+      const int head = item / half;
+      const int pair = item - head * half;
+      float* x = prepared_row + (long)head * dh;
+      const int ia = interleaved ? 2 * pair : pair;
+      const int ib = interleaved ? 2 * pair + 1 : pair + half;
+      const float cosine = turns[2 * pair], sine = turns[2 * pair + 1];
+      const float u = x[ia], v = x[ib];
+      x[ia] = u * cosine - v * sine;
+      x[ib] = v * cosine + u * sine;
+    }
+    __syncthreads();
+  }
+  if (head_norm == 2) norm_heads();
   long cell = -1, page = 0;
   int offset = 0;
   if (slot_mapping) {
@@ -184,19 +222,10 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
     page = cell / page_size;
     offset = (int)(cell - page * page_size);
   }
-  // q heads then k heads: a thread an element; the partner of a turned element is read from LDS, which nobody writes
   for (int item = threadIdx.x; item < q_cols + k_cols; item += blockDim.x) {
     const int head = item / dh;
     const int j = item - head * dh;
-    const float* x = prepared_row + (long)head * dh;
-    float value = x[j];
-    if (inv_freq && j < rotary_dim) {
-      const bool low = j < half;
-      const int pair = low ? j : j - half;
-      const float cosine = turns[2 * pair], sine = turns[2 * pair + 1];
-      const float partner = x[low ? j + half : j - half];
-      value = low ? value * cosine - partner * sine : value * cosine + partner * sine;
-    }
+    const float value = prepared_row[item];
     if (head < Hq) row[item] = from_float<T>(value);
     else if (cell >= 0)
       k_base[page * page_stride + ((long)(head - Hq) * page_size + offset) * dh + j] = from_float<T>(value);
@@ -220,7 +249,9 @@ attention_prepare_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, 
 
 extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq, int Hkv, int dh, int dv,
                                     int values_from_keys, const int* positions, const float* inv_freq, int rotary_dim,
+                                    int interleaved, float turn_scale,
                                     const float* q_norm, const float* k_norm, float norm_eps,
+                                    int head_norm, const float* q_head_weight, const float* k_head_weight, float head_eps,
                                     const float* value_inv_freq, const int* slot_mapping, void* k_base, void* v_base,
                                     long page_stride, int page_size, hipStream_t stream) {
   if (!qkv || !positions || T <= 0 || Hq <= 0 || Hkv <= 0 || dh <= 0 || dv <= 0) return ERR_BAD_ARGUMENT;
@@ -228,6 +259,8 @@ extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq
   if (values_from_keys && dv != dh) return ERR_BAD_ARGUMENT;
   if (value_inv_freq && (dv & 1)) return ERR_BAD_ARGUMENT;
   if ((q_norm == nullptr) != (k_norm == nullptr)) return ERR_BAD_ARGUMENT;
+  if (head_norm < 0 || head_norm > 2 || (head_norm && q_norm) || (head_norm && !(head_eps > 0.f))) return ERR_BAD_ARGUMENT;
+  if ((q_head_weight == nullptr) != (k_head_weight == nullptr) || (q_head_weight && !head_norm)) return ERR_BAD_ARGUMENT;
   if (ld < (long)(Hq + Hkv) * dh + (values_from_keys ? 0L : (long)Hkv * dv)) return ERR_BAD_ARGUMENT;
   if (slot_mapping && (!k_base || !v_base || page_size <= 0)) return ERR_BAD_ARGUMENT;
   if (!inv_freq) rotary_dim = 0;
@@ -236,14 +269,16 @@ extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq
   if (lds > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   if (dtype == DT_F32)
     attention_prepare_kernel<float><<<T, 256, lds, stream>>>((float*)qkv, ld, Hq, Hkv, dh, dv, values_from_keys, positions,
-                                                             inv_freq, rotary_dim, q_norm, k_norm, norm_eps,
+                                                             inv_freq, rotary_dim, interleaved, turn_scale, q_norm, k_norm,
+                                                             norm_eps, head_norm, q_head_weight, k_head_weight, head_eps,
                                                              value_inv_freq, slot_mapping, (float*)k_base, (float*)v_base,
                                                              page_stride, page_size);
   else if (dtype == DT_BF16)
     attention_prepare_kernel<bf16_t><<<T, 256, lds, stream>>>((bf16_t*)qkv, ld, Hq, Hkv, dh, dv, values_from_keys,
-                                                              positions, inv_freq, rotary_dim, q_norm, k_norm, norm_eps,
-                                                              value_inv_freq, slot_mapping, (bf16_t*)k_base,
-                                                              (bf16_t*)v_base, page_stride, page_size);
+                                                              positions, inv_freq, rotary_dim, interleaved, turn_scale,
+                                                              q_norm, k_norm, norm_eps, head_norm, q_head_weight,
+                                                              k_head_weight, head_eps, value_inv_freq, slot_mapping,
+                                                              (bf16_t*)k_base, (bf16_t*)v_base, page_stride, page_size);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();
@@ -254,7 +289,8 @@ extern "C" int mi_attention_prepare(void* qkv, int dtype, long ld, int T, int Hq
 // Works for any head_dim <= 256, any page size, any group size, float32 and bfloat16; the float32 path of
 // the whole model uses it for prompts and for decoding alike.
 //   s = q.k * scale;  visible keys: position <= query position, and
-//   query - key < window when window > 0 (reference: src/decoder.rs:4515-4532);
+//   query - key < window when window > 0 (reference: src/decoder.rs:4515-4532); with kept > 0 the keys at
+//   positions below kept stay visible behind the window (the first tokens of a sequence, at their true positions);
 //   softmax in float32 (reference: src/decoder.rs:4665-4667).
 // `slopes` (optional, float32 per query head): a position encoding that is a bias on the scores,
 //   s -= slopes[head] * (query position - key position)   (no counterpart in the reference).
@@ -285,7 +321,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
                        const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                        int page_size, const int* __restrict__ block_tables, int max_pages,
                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
-                       int window, const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
+                       int window, int kept, const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
                        float* __restrict__ partial, const float* __restrict__ head_scales,
                        const float* __restrict__ score_bias, int sigmoid) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
@@ -301,7 +337,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   const int query_position = positions[token];
   int first_key = 0;
   if (window > 0 && query_position - window + 1 > 0) first_key = query_position - window + 1;
-  if ((run + 1) * PA_RUN <= first_key || run * PA_RUN > query_position) return;   // no key of this run is visible
+  if (((run + 1) * PA_RUN <= first_key && run * PA_RUN >= kept) || run * PA_RUN > query_position) return;   // no key of this run is visible
   const int kvh = head / (Hq / Hkv);
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
@@ -312,7 +348,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   __syncthreads();
 
   const int key = run * PA_RUN + wave * WAVE + lane;
-  const bool visible = key >= first_key && key <= query_position;
+  const bool visible = (key >= first_key || key < kept) && key <= query_position;
   float score = -INFINITY;
   long row_offset = 0;
   int offset = 0;
@@ -348,7 +384,9 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   offset_shared[wave][lane] = offset;
   __syncthreads();
   const int wave_first = run * PA_RUN + wave * WAVE;
-  const int from = min(WAVE, max(0, first_key - wave_first));
+  // a wave that holds kept first keys walks from its start: the keys between them and the window weigh 0 and are
+  // not added (their cells may be anything)
+  const int from = wave_first < kept ? 0 : min(WAVE, max(0, first_key - wave_first));
   const int to = min(WAVE, max(0, query_position - wave_first + 1));
   if (lane == 0) {
     // the normalizer: the probabilities added up in the order of their keys (a sum whose order the keys fix,
@@ -375,8 +413,9 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
-          const float added = fmaf(p_shared[wave][min(j0 + u, WAVE - 1)], values[u], sum);
-          sum = j0 + u < to ? added : sum;
+          const float weight_u = p_shared[wave][min(j0 + u, WAVE - 1)];
+          const float added = fmaf(weight_u, values[u], sum);
+          sum = (j0 + u < to && (kept <= 0 || weight_u != 0.f)) ? added : sum;
         }
       }
       wave_o[wave][dim] = sum;
@@ -447,7 +486,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
                             const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                             int page_size, const int* __restrict__ block_tables, int max_pages,
                             const int* __restrict__ query_tiles, int tile_tokens, const int* __restrict__ cu_seqlens,
-                            const int* __restrict__ positions, float scale, int window,
+                            const int* __restrict__ positions, float scale, int window, int kept,
                             const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
                             float* __restrict__ partial, const float* __restrict__ head_scales,
                             const float* __restrict__ score_bias, int sigmoid) {
@@ -475,7 +514,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
   const int first_position = positions[first_row];
   int tile_first_key = 0;                                           // the oldest key any query of the tile sees
   if (window > 0 && first_position - window + 1 > 0) tile_first_key = first_position - window + 1;
-  if (run * PA_RUN > last_position || (run + 1) * PA_RUN <= tile_first_key) return;
+  if (run * PA_RUN > last_position || ((run + 1) * PA_RUN <= tile_first_key && run * PA_RUN >= kept)) return;
   const int kvh = head / (Hq / Hkv);
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
@@ -507,7 +546,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
   auto take_group = [&](auto group_constant) {
     constexpr int g = decltype(group_constant)::value;
     const int group_first = run * PA_RUN + g * WAVE;
-    if (group_first > last_position || group_first + WAVE <= tile_first_key) return;       // the same for every thread
+    if (group_first > last_position || (group_first + WAVE <= tile_first_key && group_first >= kept)) return;       // the same for every thread
     __syncthreads();                                    // the group before is read (and the queries are laid down)
     // keys group_first .. group_first + 63 that some query of the tile sees; the others (cells never written,
     // pages the request does not hold) are not fetched and lie in LDS as zeros that nobody multiplies
@@ -519,7 +558,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       const int quarter = dh >> 2;
       const int dim0 = (tid & 3) * quarter;
       float* to = k_lds + key_in * k_ld + dim0;
-      if (key_in < keys && key_in >= skipped) {
+      if (key_in < keys && (key_in >= skipped || group_first + key_in < kept)) {
         const int key = group_first + key_in;
         const int page = table[key / page_size];
         const T* from = k_base + (long)page * page_stride + ((long)kvh * page_size + key % page_size) * dh + dim0;
@@ -535,7 +574,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
     {
       // values: a thread a key (the lanes of a wave walk along a page's tokens), the waves take every fourth dim
       const int key_in = lane;
-      if (key_in < keys && key_in >= skipped) {
+      if (key_in < keys && (key_in >= skipped || group_first + key_in < kept)) {
         const int key = group_first + key_in;
         const int page = table[key / page_size];
         const T* from = v_base + (long)page * page_stride + (long)kvh * dv * page_size + key % page_size;
@@ -573,7 +612,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       int first_key = 0;
       if (window > 0 && position - window + 1 > 0) first_key = position - window + 1;
       const int key = group_first + lane;
-      const bool visible = key >= first_key && key <= position;
+      const bool visible = (key >= first_key || key < kept) && key <= position;
       float score = -INFINITY;
       if (visible) {
         score = dot[i] * scale;
@@ -651,7 +690,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
     const int position = query_position[i];
     int first_key = 0;
     if (window > 0 && position - window + 1 > 0) first_key = position - window + 1;
-    if (position < 0 || (run + 1) * PA_RUN <= first_key || run * PA_RUN > position) continue;    // the per-token kernel writes nothing either
+    if (position < 0 || ((run + 1) * PA_RUN <= first_key && run * PA_RUN >= kept) || run * PA_RUN > position) continue;    // the per-token kernel writes nothing either
     float best = group_max[i][0];
 #pragma unroll
     for (int g = 1; g < PA_WAVES; ++g) best = fmaxf(best, group_max[i][g]);
@@ -683,9 +722,9 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
 
 template <typename T, bool FAST_EXP>
 __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, int Hq, int dh, int runs,
-                                             const int* __restrict__ positions, int window,
-                                             const float* __restrict__ sinks, T* __restrict__ out, long out_ld,
-                                             int sigmoid) {
+                                             const int* __restrict__ positions, int window, int kept,
+                                             const float* __restrict__ sinks, float fixed_sink, int has_fixed_sink,
+                                             T* __restrict__ out, long out_ld, int sigmoid) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int query_position = positions[token];
@@ -698,7 +737,8 @@ __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, 
   const float* theirs = partial + ((token * Hq + head) * runs) * (long)(dh + 2);
   for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
     float maximum = -INFINITY, denominator = 0.f, sum = 0.f;
-    for (int run = first_run; run <= last_run; ++run) {
+    for (int run = 0; run <= last_run; ++run) {
+      if (run < first_run && run * PA_RUN >= kept) continue;       // behind the window and past the kept first keys: never written
       const float* one = theirs + (long)run * (dh + 2);
       const float larger = fmaxf(maximum, one[0]);
       const float keep = FAST_EXP ? __expf(maximum - larger) : expf(maximum - larger);     // 0 the first time
@@ -707,9 +747,9 @@ __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, 
       sum = sum * keep + weight * one[2 + dim];
       maximum = larger;
     }
-    if (sinks) {
+    if (sinks || has_fixed_sink) {
       // the sink: a term of the denominator that brings no value
-      const float sink = sinks[head];
+      const float sink = sinks ? sinks[head] : fixed_sink;
       const float larger = fmaxf(maximum, sink);
       const float keep = FAST_EXP ? __expf(maximum - larger) : expf(maximum - larger);
       denominator = denominator * keep + (FAST_EXP ? __expf(sink - larger) : expf(sink - larger));
@@ -756,13 +796,14 @@ static int raise_tile_lds(size_t bytes) {
 extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh, int dv,
                                   const void* k_base, const void* v_base, long page_stride, int page_size,
                                   const int* block_tables, int max_pages, const int* lane_of_token,
-                                  const int* positions, float scale, int window, const float* slopes,
-                                  const float* log_bias, const float* sinks,
+                                  const int* positions, float scale, int window, int kept, const float* slopes,
+                                  const float* log_bias, const float* sinks, float fixed_sink, int has_fixed_sink,
                                   int max_seq_len, float* partial, long partial_floats, void* out, long out_ld,
                                   const int* query_tiles, int num_tiles, int tile_tokens, const int* cu_seqlens,
                                   const float* head_scales, const float* score_bias, int sigmoid,
                                   hipStream_t stream) {
-  if ((score_bias && !sigmoid) || (sigmoid && sinks)) return ERR_BAD_ARGUMENT;
+  if ((score_bias && !sigmoid) || (sigmoid && (sinks || has_fixed_sink)) || (sinks && has_fixed_sink)) return ERR_BAD_ARGUMENT;
+  if (kept < 0 || (kept > 0 && window <= 0)) return ERR_BAD_ARGUMENT;
   if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || dv <= 0 || page_size <= 0 || max_pages <= 0 ||
       max_seq_len <= 0 || !partial)
     return ERR_BAD_ARGUMENT;
@@ -795,7 +836,7 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
 #define TILE_LAUNCH(T_, FAST_, DIMS_)                                                                                 \
   paged_attention_tile_kernel<T_, FAST_, DIMS_><<<tile_grid, PA_RUN, tile_lds, stream>>>(                              \
       (const T_*)q, q_ld, Hq, Hkv, dh, dv, (const T_*)k_base, (const T_*)v_base, page_stride, page_size, block_tables, \
-      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, log_bias, runs, partial,       \
+      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, kept, slopes, log_bias, runs, partial, \
       head_scales, score_bias, sigmoid)
     if (tiled && dims == 1) TILE_LAUNCH(float, false, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(float, false, 2);
@@ -803,11 +844,11 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
     else
       paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
           (const float*)q, q_ld, Hq, Hkv, dh, dv, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial,
+          block_tables, max_pages, lane_of_token, positions, scale, window, kept, slopes, log_bias, runs, partial,
           head_scales, score_bias, sigmoid);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dv, runs, positions, window, sinks, (float*)out, out_ld, sigmoid);
+        partial, Hq, dv, runs, positions, window, kept, sinks, fixed_sink, has_fixed_sink, (float*)out, out_ld, sigmoid);
   } else if (dtype == DT_BF16) {
     if (tiled && dims == 1) TILE_LAUNCH(bf16_t, true, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(bf16_t, true, 2);
@@ -815,11 +856,11 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
     else
       paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
           (const bf16_t*)q, q_ld, Hq, Hkv, dh, dv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial,
-          head_scales, score_bias, sigmoid);
+          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, kept, slopes, log_bias, runs,
+          partial, head_scales, score_bias, sigmoid);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dv, runs, positions, window, sinks, (bf16_t*)out, out_ld, sigmoid);
+        partial, Hq, dv, runs, positions, window, kept, sinks, fixed_sink, has_fixed_sink, (bf16_t*)out, out_ld, sigmoid);
   } else {
     return ERR_BAD_ARGUMENT;
   }

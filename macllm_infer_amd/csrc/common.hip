@@ -266,6 +266,74 @@ extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, 
   return 0;
 }
 
+// ---------------------------------------------------------------- branches normed each on its own, then summed
+// out[r] = sum over the branches b (in their order) of factor_b * x_b[r] / sqrt(mean(x_b[r]^2) + eps_b) * weight_b,
+// float32: the outputs of a layer's mixers, each through an RMS norm of its own, before they join the stream.
+// One workgroup a row; a branch's sum of squares is a float32 sum whose order the width alone fixes.
+#define NORMED_SUM_MOST 4
+struct NormedSumBranches {
+  const void* rows[NORMED_SUM_MOST];
+  const float* weight[NORMED_SUM_MOST];
+  float factor[NORMED_SUM_MOST];
+  float eps[NORMED_SUM_MOST];
+  int is_bf16[NORMED_SUM_MOST];
+  long ld[NORMED_SUM_MOST];
+};
+
+__global__ void __launch_bounds__(256)
+normed_sum_kernel(NormedSumBranches branches, int count, float* __restrict__ out, int d) {
+  __shared__ float scratch[16];
+  const long row = blockIdx.x;
+  float scale[NORMED_SUM_MOST];
+  for (int b = 0; b < count; ++b) {
+    float squares = 0.f;
+    if (branches.is_bf16[b]) {
+      const bf16_t* x = (const bf16_t*)branches.rows[b] + row * branches.ld[b];
+      for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = to_float(x[i]);
+        squares = fmaf(v, v, squares);
+      }
+    } else {
+      const float* x = (const float*)branches.rows[b] + row * branches.ld[b];
+      for (int i = threadIdx.x; i < d; i += blockDim.x) squares = fmaf(x[i], x[i], squares);
+    }
+    const float total = block_sum(squares, scratch);
+    scale[b] = 1.0f / sqrtf(total / (float)d + branches.eps[b]);
+  }
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float sum = 0.f;
+    for (int b = 0; b < count; ++b) {
+      const float v = branches.is_bf16[b] ? to_float(((const bf16_t*)branches.rows[b])[row * branches.ld[b] + i])
+                                          : ((const float*)branches.rows[b])[row * branches.ld[b] + i];
+      sum = fmaf(branches.factor[b], v * scale[b] * branches.weight[b][i], sum);
+    }
+    out[row * d + i] = sum;
+  }
+}
+
+extern "C" int mi_normed_sum(const void* const* rows, const int* dtypes, const long* lds, const float* const* weights,
+                             const float* factors, const float* eps, int count, float* out, int T, int d,
+                             hipStream_t stream) {
+  if (!rows || !dtypes || !lds || !weights || !factors || !eps || !out || count <= 0 || T <= 0 || d <= 0)
+    return ERR_BAD_ARGUMENT;
+  if (count > NORMED_SUM_MOST) return ERR_UNSUPPORTED_SIZE;
+  NormedSumBranches branches;
+  for (int b = 0; b < NORMED_SUM_MOST; ++b) {
+    const int from = b < count ? b : 0;
+    if (!rows[from] || !weights[from] || lds[from] < d || !(eps[from] > 0.f)) return ERR_BAD_ARGUMENT;
+    if (dtypes[from] != DT_F32 && dtypes[from] != DT_BF16) return ERR_BAD_ARGUMENT;
+    branches.rows[b] = rows[from];
+    branches.weight[b] = weights[from];
+    branches.factor[b] = factors[from];
+    branches.eps[b] = eps[from];
+    branches.is_bf16[b] = dtypes[from] == DT_BF16;
+    branches.ld[b] = lds[from];
+  }
+  normed_sum_kernel<<<T, 256, 0, stream>>>(branches, count, out, d);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 // ---------------------------------------------------------------- SwiGLU
 // out[t, i] = SiLU(g[t, i]) * u[t, i]      (reference: src/decoder.rs:298-305)
 // A row of the input holds [g | u] (tile = 0), or g and u interleaved in tiles:

@@ -77,6 +77,7 @@ struct Table {
 struct Group {
   int page_size;
   int window;               // <= 0: every key is kept
+  int kept_first = 0;       // with a window: keys at positions below this stay visible, their pages are never given back
   Pool pool;
   std::vector<Table> tables;   // by slot
   Group(int page_size_, int pages, int window_, int slots)
@@ -119,6 +120,13 @@ void* hc_create(int num_groups, const int* page_size, const int* num_pages, cons
   core->groups.reserve(num_groups);
   for (int g = 0; g < num_groups; ++g) core->groups.emplace_back(page_size[g], num_pages[g], window[g], max_slots);
   return core;
+}
+// A group whose window also keeps the first `tokens` keys of every request: the pages that hold them stay.
+int hc_keep_first(void* handle, int group, int tokens) {
+  Core* core = (Core*)handle;
+  if (group < 0 || group >= (int)core->groups.size() || tokens < 0) return -1;
+  core->groups[group].kept_first = tokens;
+  return 0;
 }
 void hc_destroy(void* core) { delete (Core*)core; }
 void* hc_group_pool(void* core, int group) { return &((Core*)core)->groups[group].pool; }
@@ -220,9 +228,12 @@ int hc_commit(void* handle, int n, const int* slots, const int* tokens) {
       const long first_needed_key = (long)core->length[slot] - group.window + 1;
       if (first_needed_key <= 0) continue;
       const int first_needed_page = (int)std::min<long>(first_needed_key / group.page_size, (long)table.pages.size());
-      if (first_needed_page <= table.first_live) continue;
-      if (!group.pool.give(table.pages.data() + table.first_live, first_needed_page - table.first_live)) return -2;
-      for (int page = table.first_live; page < first_needed_page; ++page) table.pages[page] = -1;
+      // the pages of the kept first keys are never passed: what is given back starts behind them
+      const int kept_pages = (group.kept_first + group.page_size - 1) / group.page_size;
+      const int from = std::max(table.first_live, kept_pages);
+      if (first_needed_page <= from) continue;
+      if (!group.pool.give(table.pages.data() + from, first_needed_page - from)) return -2;
+      for (int page = from; page < first_needed_page; ++page) table.pages[page] = -1;
       table.first_live = first_needed_page;
     }
   }

@@ -90,7 +90,8 @@ extern "C" int mi_latent_prepare(const void* down, int dtype, long ld, int T, in
                                  const float* inv_freq, int rotary_dim, int interleaved, const int* slot_mapping,
                                  void* k_cache, void* v_cache, long page_stride, int page_size, void* q_latent, long q_ld,
                                  hipStream_t stream) {
-  if (!down || !q_norm || !kv_norm || !positions || !q_latent || T <= 0 || q_rank <= 0 || kv_rank <= 0 || rope_dim < 0 ||
+  // q_rank 0: the row holds no query latent (queries projected directly); q_norm and q_latent are then not read
+  if (!down || !kv_norm || !positions || T <= 0 || q_rank < 0 || (q_rank > 0 && (!q_norm || !q_latent)) || kv_rank <= 0 || rope_dim < 0 ||
       ld < q_rank + kv_rank + rope_dim || q_ld < q_rank || rotary_dim < 0 || rotary_dim > rope_dim || rotary_dim % 2 ||
       (rotary_dim > 0 && !inv_freq) || (slot_mapping && (!k_cache || !v_cache || page_size <= 0)))
     return ERR_BAD_ARGUMENT;

@@ -13,6 +13,7 @@
 #define CONV_MAX_K 16
 
 // ---------------------------------------------------------------- conv + SiLU
+// (activation 1: SiLU of the sum; 0: the sum as it is, for a convolution with nothing behind it)
 // c[t, ch] = bias[ch] + sum_k w[ch, k] * win[t + k, ch], win = [tail ; this lane's rows];
 // w[ch, 0] multiplies the oldest sample (reference: src/decoder.rs:2233-2253, :5948-5950).
 template <typename T>
@@ -20,7 +21,7 @@ __global__ void conv1d_silu_kernel(const T* __restrict__ u, long ld, int col_off
                                    const float* __restrict__ weight, const float* __restrict__ bias,
                                    const T* __restrict__ conv_state, const int* __restrict__ lane_of_token,
                                    const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
-                                   T* __restrict__ out, long total) {
+                                   T* __restrict__ out, long total, int activation) {
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (index >= total) return;
   const long token = index / C;
@@ -38,7 +39,7 @@ __global__ void conv1d_silu_kernel(const T* __restrict__ u, long ld, int col_off
       sample = to_float(tail[((K - 1) + (source - lane_start)) * C + channel]);
     sum += weight[channel * K + k] * sample;
   }
-  out[index] = from_float<T>(silu_f(sum));
+  out[index] = from_float<T>(activation ? silu_f(sum) : sum);
 }
 
 // The same for float32 with four neighbouring channels a thread (16-byte loads of the rows, the taps of the four
@@ -49,7 +50,7 @@ conv1d_silu_f32x4_kernel(const float* __restrict__ u, long ld, int col_offset, i
                          const float* __restrict__ weight, const float* __restrict__ bias,
                          const float* __restrict__ conv_state, const int* __restrict__ lane_of_token,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
-                         float* __restrict__ out, long total) {
+                         float* __restrict__ out, long total, int activation) {
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (index >= total) return;
   const int vectors = C / 4;
@@ -80,7 +81,7 @@ conv1d_silu_f32x4_kernel(const float* __restrict__ u, long ld, int col_offset, i
     float sum = bias ? bias[channel + c] : 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k) sum += taps[c * K + k] * reinterpret_cast<const float*>(&window[k])[c];
-    results[c] = silu_f(sum);
+    results[c] = activation ? silu_f(sum) : sum;
   }
   *reinterpret_cast<float4*>(out + token * (long)C + channel) = result;
 }
@@ -99,7 +100,7 @@ conv1d_silu_vec_kernel(const bf16_t* __restrict__ u, long ld, int col_offset, in
                        const float* __restrict__ weight, const float* __restrict__ bias,
                        const bf16_t* __restrict__ conv_state, const int* __restrict__ lane_of_token,
                        const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
-                       bf16_t* __restrict__ out) {
+                       bf16_t* __restrict__ out, int activation) {
   constexpr int ROWS = 4;
   const int vectors = C / 8;
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -154,7 +155,7 @@ conv1d_silu_vec_kernel(const bf16_t* __restrict__ u, long ld, int col_offset, in
     }
     conv_bf16x8 result;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) result[c] = (bf16_t)silu_f(sum[c]);
+    for (int c = 0; c < 8; ++c) result[c] = (bf16_t)(activation ? silu_f(sum[c]) : sum[c]);
     *reinterpret_cast<conv_bf16x8*>(out + token * C + channel) = result;
   }
 }
@@ -162,7 +163,7 @@ conv1d_silu_vec_kernel(const bf16_t* __restrict__ u, long ld, int col_offset, in
 extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset, int T, int C, int K,
                               const float* weight, const float* bias, const void* conv_state,
                               const int* lane_of_token, const int* cu_seqlens, const int* slot_ids, void* out,
-                              hipStream_t stream) {
+                              int activation, hipStream_t stream) {
   if (T <= 0 || C <= 0 || K <= 0 || K > CONV_MAX_K || ld < col_offset + C) return ERR_BAD_ARGUMENT;
   const long total = (long)T * C;
   const int blocks = (int)((total + 255) / 256);
@@ -175,7 +176,7 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
 #define CONV_CASE(K_)                                                                                          \
   conv1d_silu_vec_kernel<K_><<<vec_blocks, 256, 0, stream>>>((const bf16_t*)u, ld, col_offset, C, T, weight,   \
                                                              bias, (const bf16_t*)conv_state, lane_of_token,   \
-                                                             cu_seqlens, slot_ids, (bf16_t*)out)
+                                                             cu_seqlens, slot_ids, (bf16_t*)out, activation)
     if (K == 2) CONV_CASE(2);
     else if (K == 3) CONV_CASE(3);
     else CONV_CASE(4);
@@ -191,7 +192,7 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
 #define CONV_F32_CASE(K_)                                                                                        \
   conv1d_silu_f32x4_kernel<K_><<<vec_blocks, 256, 0, stream>>>((const float*)u, ld, col_offset, C, weight, bias, \
                                                                (const float*)conv_state, lane_of_token,          \
-                                                               cu_seqlens, slot_ids, (float*)out, threads)
+                                                               cu_seqlens, slot_ids, (float*)out, threads, activation)
     if (K == 2) CONV_F32_CASE(2);
     else if (K == 3) CONV_F32_CASE(3);
     else CONV_F32_CASE(4);
@@ -202,11 +203,11 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
   if (dtype == DT_F32)
     conv1d_silu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)u, ld, col_offset, C, K, weight, bias,
                                                            (const float*)conv_state, lane_of_token, cu_seqlens,
-                                                           slot_ids, (float*)out, total);
+                                                           slot_ids, (float*)out, total, activation);
   else if (dtype == DT_BF16)
     conv1d_silu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)u, ld, col_offset, C, K, weight, bias,
                                                             (const bf16_t*)conv_state, lane_of_token, cu_seqlens,
-                                                            slot_ids, (bf16_t*)out, total);
+                                                            slot_ids, (bf16_t*)out, total, activation);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();
@@ -265,7 +266,7 @@ extern "C" int mi_conv_state_update(const void* u, int dtype, long ld, int col_o
 template <typename T, int MAXK>
 __global__ void conv_step_kernel(T* __restrict__ u, long ld, int col_offset, int C, int K, const float* __restrict__ weight,
                                  const float* __restrict__ bias, T* __restrict__ conv_state,
-                                 const int* __restrict__ slot_ids, long total) {
+                                 const int* __restrict__ slot_ids, long total, int activation) {
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (index >= total) return;
   const int m = (int)(index / C);
@@ -291,17 +292,18 @@ __global__ void conv_step_kernel(T* __restrict__ u, long ld, int col_offset, int
     }
   }
   if (K > 1) tail[(long)(K - 2) * C] = sample;
-  *cell = (T)silu_f(sum);
+  *cell = (T)(activation ? silu_f(sum) : sum);
 }
 
 extern "C" int mi_conv_step(void* u, int dtype, long ld, int col_offset, int M, int C, int K, const float* weight,
-                            const float* bias, void* conv_state, const int* slot_ids, hipStream_t stream) {
+                            const float* bias, void* conv_state, const int* slot_ids, int activation,
+                            hipStream_t stream) {
   if (M <= 0 || C <= 0 || K <= 0 || K > CONV_MAX_K) return ERR_BAD_ARGUMENT;
   const long total = (long)M * C;
   const int blocks = (int)((total + 255) / 256);
 #define CONV_STEP(T_, MAXK_)                                                                                  \
   conv_step_kernel<T_, MAXK_><<<blocks, 256, 0, stream>>>((T_*)u, ld, col_offset, C, K, weight, bias, (T_*)conv_state, \
-                                                          slot_ids, total)
+                                                          slot_ids, total, activation)
   if (dtype == DT_F32) {
     if (K <= 4) CONV_STEP(float, 4);
     else CONV_STEP(float, CONV_MAX_K);

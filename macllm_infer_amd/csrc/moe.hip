@@ -1,7 +1,8 @@
 // A feed-forward of many small experts of which a token uses a few.
 //
 //   moe_route        float32 router logits -> softmax, correction, the token's experts and their weights (one wave
-//                    a token), and the sigmoid of the shared expert's gate logit
+//                    a token), and the sigmoid of the shared expert's gate logit; or (mode 1) logits + bias -> the
+//                    largest ones and the softmax over those alone
 //   moe_plan         the step's (token, choice) rows grouped by expert, every expert's rows starting a tile of 16
 //                    places: built on the device by one workgroup, so that no count has to travel to the host and
 //                    the launches that follow depend on the number of tokens alone
@@ -20,7 +21,8 @@
 // ---------------------------------------------------------------- router
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int top, const float* __restrict__ correction,
-                 float scale, float eps, int* __restrict__ chosen, float* __restrict__ weights, float* __restrict__ gate) {
+                 float scale, float eps, int mode, int* __restrict__ chosen, float* __restrict__ weights,
+                 float* __restrict__ gate) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int token = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   if (token >= T) return;
@@ -35,23 +37,35 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
     score[j] = e < E ? row[e] : -INFINITY;
     most = fmaxf(most, score[j]);
   }
-  most = wave_max(most);
-  float total = 0.f;
+  if (mode == 0) {
+    most = wave_max(most);
+    float total = 0.f;
 #pragma unroll
-  for (int j = 0; j < MOE_PER_LANE; ++j) {
-    if (j >= held) break;
-    const int e = lane + WAVE * j;
-    score[j] = e < E ? expf(score[j] - most) : 0.f;
-    total += score[j];
-  }
-  total = wave_sum(total);
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      if (j >= held) break;
+      const int e = lane + WAVE * j;
+      score[j] = e < E ? expf(score[j] - most) : 0.f;
+      total += score[j];
+    }
+    total = wave_sum(total);
 #pragma unroll
-  for (int j = 0; j < MOE_PER_LANE; ++j) {
-    if (j >= held) break;
-    const int e = lane + WAVE * j;
-    score[j] = score[j] / total;
-    choice[j] = e < E ? score[j] + correction[e] : -INFINITY;
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      if (j >= held) break;
+      const int e = lane + WAVE * j;
+      score[j] = score[j] / total;
+      choice[j] = e < E ? score[j] + correction[e] : -INFINITY;
+    }
+  } else {
+    // the logits with their bias are what is chosen by and what is weighted
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      if (j >= held) break;
+      const int e = lane + WAVE * j;
+      score[j] = e < E ? score[j] + correction[e] : -INFINITY;
+      choice[j] = score[j];
+    }
   }
+  float first_picked = 0.f;        // mode 1: the largest chosen logit, which is the first one picked
   float picked_sum = 0.f;
   float mine = 0.f;            // lane k keeps the score of the k-th choice
   int mine_id = 0;
@@ -82,6 +96,10 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
 #pragma unroll
     for (int j = 0; j < MOE_PER_LANE; ++j)
       if (j < held && lane + WAVE * j == best_id) choice[j] = -INFINITY;
+    if (mode != 0) {
+      if (k == 0) first_picked = best_score;
+      best_score = expf(best_score - first_picked);
+    }
     picked_sum += best_score;
     if ((k & (WAVE - 1)) == lane) {
       // more choices than lanes: written as they come
@@ -105,12 +123,15 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
   if (gate && lane == 0) gate[token] = 1.0f / (1.0f + expf(-row[E]));
 }
 
+// mode 0: softmax over all experts, choice by score + correction, weights score / (sum of the chosen + eps) * scale.
+// mode 1: choice by logit + correction (a bias), weights the softmax over the chosen (logit + correction) * scale.
 extern "C" int mi_moe_route(const float* logits, long ld, int T, int E, int top, const float* correction, float scale,
-                            float eps, int* chosen, float* weights, float* gate, hipStream_t stream) {
+                            float eps, int mode, int* chosen, float* weights, float* gate, hipStream_t stream) {
   if (!logits || !correction || !chosen || !weights || T <= 0 || E <= 0 || top <= 0 || top > E || ld < E + (gate ? 1 : 0))
     return ERR_BAD_ARGUMENT;
   if (E > MOE_MAX_EXPERTS) return ERR_UNSUPPORTED_SIZE;
-  moe_route_kernel<<<(T + 3) / 4, 256, 0, stream>>>(logits, ld, T, E, top, correction, scale, eps, chosen, weights, gate);
+  if (mode != 0 && mode != 1) return ERR_BAD_ARGUMENT;
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, stream>>>(logits, ld, T, E, top, correction, scale, eps, mode, chosen, weights, gate);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -171,7 +192,7 @@ template <typename T, typename TO, bool VEC, bool GLU, int MT, int PAIRS>
 __global__ void __launch_bounds__(TILE_THREADS)
 moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride, long ldw,
                        int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert, int gather,
-                       float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+                       float limit, float alpha, float offset, int squared_relu, TO* __restrict__ out, long ldo) {
   __shared__ float red[TILE_WAVES][256];
   const int tile = blockIdx.y;
   const int expert = tile_expert[tile];
@@ -209,6 +230,9 @@ moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* _
         const float g = fminf(value, limit);
         const float u = fminf(fmaxf(up, -limit), limit);
         value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+      } else if (squared_relu) {
+        value = fmaxf(value, 0.f);
+        value *= value;
       }
       const long n = n0 + 16 * p + 4 * (l / 16) + tid / 64;
       const int place = (tile * MT + mt) * 16 + (l % 16);
@@ -230,7 +254,8 @@ template <typename T, typename TO, bool GLU>
 __global__ void __launch_bounds__(TILE_THREADS)
 moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride,
                             long ldw, int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert,
-                            int gather, float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+                            int gather, float limit, float alpha, float offset, int squared_relu, TO* __restrict__ out,
+                            long ldo) {
   typedef typename TileTraits<T>::Piece Piece;
   constexpr int CHUNK = TileTraits<T>::CHUNK;
   constexpr int PIECE = TileTraits<T>::PIECE;
@@ -315,7 +340,12 @@ moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt) {
           const long n = n0 + 32 * wave + 16 * nt + 4 * q + i;
-          if (n < width) row[n] = from_float<TO>(live ? acc[nt][mt][i] : 0.f);
+          float value = acc[nt][mt][i];
+          if (squared_relu) {
+            value = fmaxf(value, 0.f);
+            value *= value;
+          }
+          if (n < width) row[n] = from_float<TO>(live ? value : 0.f);
         }
       }
     }
@@ -329,7 +359,8 @@ template <typename T, typename TO, bool GLU>
 __global__ void __launch_bounds__(TILE_THREADS)
 moe_expert_gemm_widest_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride,
                               long ldw, int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert,
-                              int gather, float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+                              int gather, float limit, float alpha, float offset, int squared_relu, TO* __restrict__ out,
+                              long ldo) {
   typedef typename TileTraits<T>::Piece Piece;
   constexpr int CHUNK = TileTraits<T>::CHUNK;
   constexpr int PIECE = TileTraits<T>::PIECE;
@@ -425,7 +456,12 @@ moe_expert_gemm_widest_kernel(const T* __restrict__ x, long ldx, int x_rows, con
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) {
           const long n = n0 + 64 * wn + 16 * nt + 4 * q + i;
-          if (n < width) row[n] = from_float<TO>(live ? acc[nt][mt][i] : 0.f);
+          float value = acc[nt][mt][i];
+          if (squared_relu) {
+            value = fmaxf(value, 0.f);
+            value *= value;
+          }
+          if (n < width) row[n] = from_float<TO>(live ? value : 0.f);
         }
       }
     }
@@ -434,30 +470,32 @@ moe_expert_gemm_widest_kernel(const T* __restrict__ x, long ldx, int x_rows, con
 
 template <typename T, typename TO>
 static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, long expert_stride, long ldw, int N, int K,
-                               const int* source, const int* tile_expert, int tiles, int pad, int gather, int glu,
+                               const int* source, const int* tile_expert, int tiles, int pad, int gather, int activation,
                                float limit, float alpha, float offset, TO* out, long ldo, hipStream_t stream) {
+  const int glu = activation == 1;
+  const int squared_relu = activation == 2;
   constexpr int PIECE = TileTraits<T>::PIECE;
   const bool vec = K % PIECE == 0 && ldx % PIECE == 0 && ldw % PIECE == 0 && expert_stride % PIECE == 0 &&
                    ((unsigned long long)x % 16) == 0 && ((unsigned long long)W % 16) == 0;
   const int width = glu ? N / 2 : N;
-#define EXPERT_LAUNCH(VEC_, GLU_, MT_, PAIRS_)                                                                           moe_expert_gemm_kernel<T, TO, VEC_, GLU_, MT_, PAIRS_>                                                                    <<<dim3((unsigned)((width + 16 * PAIRS_ - 1) / (16 * PAIRS_)), (unsigned)tiles), TILE_THREADS, 0, stream>>>(               x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
+#define EXPERT_LAUNCH(VEC_, GLU_, MT_, PAIRS_)                                                                           moe_expert_gemm_kernel<T, TO, VEC_, GLU_, MT_, PAIRS_>                                                                    <<<dim3((unsigned)((width + 16 * PAIRS_ - 1) / (16 * PAIRS_)), (unsigned)tiles), TILE_THREADS, 0, stream>>>(               x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, squared_relu, out, ldo)
 #define EXPERT_SHAPE(MT_, PAIRS_GLU_, PAIRS_PLAIN_)                                                                      do {                                                                                                                    if (vec && glu) EXPERT_LAUNCH(true, true, MT_, PAIRS_GLU_);                                                            else if (vec) EXPERT_LAUNCH(true, false, MT_, PAIRS_PLAIN_);                                                           else if (glu) EXPERT_LAUNCH(false, true, MT_, PAIRS_GLU_);                                                             else EXPERT_LAUNCH(false, false, MT_, PAIRS_PLAIN_);                                                                 } while (0)
   if (pad == 128) {      // (only plans of rows and matrices in whole pieces are made so wide)
     const dim3 grid((unsigned)((width + (glu ? 64 : 128) - 1) / (glu ? 64 : 128)), (unsigned)tiles);
     if (glu)
       moe_expert_gemm_widest_kernel<T, TO, true><<<grid, TILE_THREADS, 0, stream>>>(
-          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, squared_relu, out, ldo);
     else
       moe_expert_gemm_widest_kernel<T, TO, false><<<grid, TILE_THREADS, 0, stream>>>(
-          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, squared_relu, out, ldo);
   } else if (pad == 64 && vec) {
     const dim3 grid((unsigned)((width + (glu ? 64 : 128) - 1) / (glu ? 64 : 128)), (unsigned)tiles);
     if (glu)
       moe_expert_gemm_wide_kernel<T, TO, true><<<grid, TILE_THREADS, 0, stream>>>(
-          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, squared_relu, out, ldo);
     else
       moe_expert_gemm_wide_kernel<T, TO, false><<<grid, TILE_THREADS, 0, stream>>>(
-          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, squared_relu, out, ldo);
   } else if (pad == 64) {
     EXPERT_SHAPE(4, 2, 4);
   } else {
@@ -469,8 +507,11 @@ static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, lon
 
 extern "C" int mi_moe_expert_gemm(const void* x, int dtype, long ldx, int x_rows, const void* W, long expert_stride,
                                   long ldw, int N, int K, const int* source, const int* tile_expert, int tiles, int pad,
-                                  int gather, int glu, float limit, float alpha, float offset, void* out, int out_dtype,
-                                  long ldo, hipStream_t stream) {
+                                  int gather, int activation, float limit, float alpha, float offset, void* out,
+                                  int out_dtype, long ldo, hipStream_t stream) {
+  // activation: 0 none, 1 the clamped gated one (the matrix holds gate rows then up rows), 2 max(z, 0)^2
+  const int glu = activation == 1;
+  if (activation < 0 || activation > 2) return ERR_BAD_ARGUMENT;
   if (!x || !W || !source || !tile_expert || !out || x_rows <= 0 || N <= 0 || K <= 0 || tiles <= 0 || ldx < K || ldw < K ||
       (glu && N % 2) || ldo < (glu ? N / 2 : N))
     return ERR_BAD_ARGUMENT;
@@ -483,13 +524,13 @@ extern "C" int mi_moe_expert_gemm(const void* x, int dtype, long ldx, int x_rows
   }
   if (dtype == DT_F32 && out_dtype == DT_F32)
     launch_expert_gemm<float, float>((const float*)x, ldx, x_rows, (const float*)W, expert_stride, ldw, N, K, source,
-                                     tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+                                     tile_expert, tiles, pad, gather, activation, limit, alpha, offset, (float*)out, ldo, stream);
   else if (dtype == DT_BF16 && out_dtype == DT_BF16)
     launch_expert_gemm<bf16_t, bf16_t>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
-                                       tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (bf16_t*)out, ldo, stream);
+                                       tile_expert, tiles, pad, gather, activation, limit, alpha, offset, (bf16_t*)out, ldo, stream);
   else if (dtype == DT_BF16 && out_dtype == DT_F32)
     launch_expert_gemm<bf16_t, float>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
-                                      tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+                                      tile_expert, tiles, pad, gather, activation, limit, alpha, offset, (float*)out, ldo, stream);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();

@@ -47,6 +47,7 @@ _SIGNATURES = {
         "mi_embed_bigram": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_long, _c_long, _c_ptr, _c_ptr, _c_ptr,
                             _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_stream_add": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_normed_sum": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_add_layernorm": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr,
                              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
                              _c_ptr],
@@ -67,7 +68,8 @@ _SIGNATURES = {
                                        _c_ptr, _c_long, _c_ptr],
     },
     "moe": {
-        "mi_moe_route": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_moe_route": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                         _c_ptr],
         "mi_moe_plan": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_moe_expert_gemm": [_c_ptr, _c_int, _c_long, _c_int, _c_ptr, _c_long, _c_long, _c_int, _c_int, _c_ptr, _c_ptr,
                                _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr, _c_int, _c_long,
@@ -93,12 +95,13 @@ _SIGNATURES = {
         "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
-                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                               _c_float, _c_int, _c_int,
                                _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                _c_ptr],
         "mi_attention_prepare": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
-                                 _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int,
-                                 _c_ptr],
+                                 _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_float,
+                                 _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
@@ -115,10 +118,11 @@ _SIGNATURES = {
     },
     "mamba2": {
         "mi_conv1d_silu": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
         "mi_conv_state_update": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                  _c_ptr],
-        "mi_conv_step": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_conv_step": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                         _c_ptr],
         "mi_ssm_scan": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr],
         "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
@@ -432,6 +436,34 @@ def stream_add(h: torch.Tensor, rows: Optional[torch.Tensor], factor: float, vec
                                           _p(vector), T, d, _stream()), "stream_add")
 
 
+NORMED_SUM_MOST = 4          # branches that ``normed_sum`` takes in one launch
+
+
+def normed_sum(branches: Sequence[tuple], out: torch.Tensor) -> None:
+    """out = sum over ``branches`` [(rows [T, d], factor, weight float32 [d], eps)], in their order, of
+    factor * rows / sqrt(mean(rows^2) + eps) * weight, float32: every branch through an RMS norm of its own."""
+    _need(0 < len(branches) <= NORMED_SUM_MOST, f"normed_sum: one to {NORMED_SUM_MOST} branches")
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.is_contiguous() and out.is_cuda,
+          "normed_sum: out must be contiguous float32 [T, d]")
+    T, d = out.shape
+    count = len(branches)
+    rows = (ctypes.c_void_p * count)()
+    weights = (ctypes.c_void_p * count)()
+    dtypes = (ctypes.c_int * count)()
+    lds = (ctypes.c_long * count)()
+    factors = (ctypes.c_float * count)()
+    epsilons = (ctypes.c_float * count)()
+    for index, (tensor, factor, weight, eps) in enumerate(branches):
+        lds[index] = _row_major(tensor, "a branch")
+        _need(tensor.shape == (T, d), "normed_sum: branches must be [T, d]")
+        _need(weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous() and weight.is_cuda,
+              "normed_sum: a weight must be float32 [d] on the GPU")
+        rows[index], weights[index], dtypes[index] = tensor.data_ptr(), weight.data_ptr(), _dt(tensor)
+        factors[index], epsilons[index] = float(factor), float(eps)
+    _check(_fn("common", "mi_normed_sum")(rows, dtypes, lds, weights, factors, epsilons, count, _p(out), T, d, _stream()),
+           "normed_sum")
+
+
 def add_layernorm(h: torch.Tensor, branches: Sequence[tuple], vector: Optional[torch.Tensor],
                   weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
                   rows: Optional[torch.Tensor] = None, branch_norm: Optional[tuple] = None) -> None:
@@ -491,10 +523,11 @@ def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, up_offset: fl
 
 
 # --------------------------------------------------------------------------- latent attention
-def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rope_dim: int, q_norm: torch.Tensor,
+def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rope_dim: int, q_norm: Optional[torch.Tensor],
                    kv_norm: torch.Tensor, eps: float, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
                    rotary_dim: int, interleaved: bool, slot_mapping: Optional[torch.Tensor],
-                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], query_latent: torch.Tensor) -> None:
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                   query_latent: Optional[torch.Tensor]) -> None:
     """From a token's down-projected row [query latent | key/value latent | key part to turn]: the query latent's
     RMS norm (times ``q_norm``) into ``query_latent``; the key/value latent's RMS norm (times ``kv_norm``) and the
     key part, its first ``rotary_dim`` dimensions turned by the token's position, into the token's cache cell: K
@@ -505,7 +538,11 @@ def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rope_dim: int,
     _need(down.shape[1] >= q_rank + kv_rank + rope_dim, "latent_prepare: the projected rows are too narrow")
     _i32(positions, "positions")
     _need(positions.numel() == T, "latent_prepare: one position per token")
+    _need(q_rank >= 0 and (q_rank > 0) == (q_norm is not None) == (query_latent is not None),
+          "latent_prepare: a query latent comes with its norm and its place, or not at all")
     for name, vector, size in (("q_norm", q_norm, q_rank), ("kv_norm", kv_norm, kv_rank)):
+        if vector is None:
+            continue
         _need(vector.dtype == torch.float32 and vector.numel() == size and vector.is_contiguous() and vector.is_cuda,
               f"latent_prepare: {name} must be float32 [{size}] on the GPU")
     turned = int(rotary_dim) if inv_freq is not None else 0
@@ -513,8 +550,11 @@ def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rope_dim: int,
     if inv_freq is not None:
         _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == turned // 2 and inv_freq.is_cuda,
               "latent_prepare: inv_freq must be float32 [rotary_dim / 2]")
-    q_ld = _row_major(query_latent, "query_latent")
-    _need(query_latent.shape == (T, q_rank) and query_latent.dtype == down.dtype, "latent_prepare: query_latent must be [T, q_rank]")
+    q_ld = 0
+    if query_latent is not None:
+        q_ld = _row_major(query_latent, "query_latent")
+        _need(query_latent.shape == (T, q_rank) and query_latent.dtype == down.dtype,
+              "latent_prepare: query_latent must be [T, q_rank]")
     page_stride, page_size = 0, 0
     if slot_mapping is not None:
         _i32(slot_mapping, "slot_mapping")
@@ -662,11 +702,14 @@ def moe_tile_rows(tokens: int, top_k: int, num_experts: int, whole_pieces: bool 
 
 
 def moe_route(logits: torch.Tensor, num_experts: int, top_k: int, correction: torch.Tensor, scale: float, eps: float,
-              shared_gate: bool):
+              shared_gate: bool, routing: str = "softmax_then_top"):
     """From float32 router logits [T, >= num_experts (+ 1)]: s = softmax over the experts; the ``top_k`` largest of
     s + correction (ties to the lower number) are the token's experts (int32 [T, top_k]), their weights (float32
     [T, top_k]) s / (sum of the chosen s + eps) * scale; with ``shared_gate`` also sigmoid of column
-    ``num_experts`` (float32 [T]), else None."""
+    ``num_experts`` (float32 [T]), else None.  ``routing`` "top_then_softmax": the ``top_k`` largest of
+    logits + correction (the correction is then a bias of the logits) are chosen, and their weights are the softmax
+    over these alone, times scale."""
+    _need(routing in ("softmax_then_top", "top_then_softmax"), f"moe_route: routing {routing!r} is not known")
     ld = _row_major(logits, "logits")
     T = logits.shape[0]
     _need(logits.dtype == torch.float32 and logits.shape[1] >= num_experts + (1 if shared_gate else 0),
@@ -678,7 +721,8 @@ def moe_route(logits: torch.Tensor, num_experts: int, top_k: int, correction: to
     weights = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
     gate = torch.empty((T,), dtype=torch.float32, device=logits.device) if shared_gate else None
     _check(_fn("moe", "mi_moe_route")(_p(logits), ld, T, num_experts, top_k, _p(correction), float(scale), float(eps),
-                                      _p(chosen), _p(weights), _p(gate), _stream()), "moe_route", f"(experts={num_experts})")
+                                      0 if routing == "softmax_then_top" else 1, _p(chosen), _p(weights), _p(gate),
+                                      _stream()), "moe_route", f"(experts={num_experts})")
     return chosen, weights, gate
 
 
@@ -708,11 +752,14 @@ def moe_plan(chosen: torch.Tensor, num_experts: int, pad: Optional[int] = None) 
     return MoePlan(chosen, num_experts, pad)
 
 
-def moe_expert_gemm(x: torch.Tensor, plan: MoePlan, weight: torch.Tensor, out: torch.Tensor, gather: bool, glu) -> None:
+def moe_expert_gemm(x: torch.Tensor, plan: MoePlan, weight: torch.Tensor, out: torch.Tensor, gather: bool, glu,
+                    squared_relu: bool = False) -> None:
     """The grouped product of a plan's rows with their experts' matrices ``weight`` [experts, N, K]: the row at a
     place is ``x[source[place]]`` (``gather``) or ``x[place]``; out[place] = weight[expert] . row, or with ``glu``
     (limit, alpha, up_offset; N = 2 I, gate rows then up rows) the clamped gated activation of the two halves,
-    [capacity, I].  Float32 sums on the matrix cores; float32 operands give a true 32-bit product."""
+    [capacity, I]; or with ``squared_relu`` max(weight[expert] . row, 0)^2.  Float32 sums on the matrix cores;
+    float32 operands give a true 32-bit product."""
+    _need(not (squared_relu and glu is not None), "moe_expert_gemm: one activation")
     ldx = _row_major(x, "x")
     ldo = _row_major(out, "out")
     _need(weight.dim() == 3 and weight.is_contiguous() and weight.is_cuda and x.dtype == weight.dtype,
@@ -723,7 +770,7 @@ def moe_expert_gemm(x: torch.Tensor, plan: MoePlan, weight: torch.Tensor, out: t
           and (not gather or x.shape[0] == plan.tokens), "moe_expert_gemm: shapes do not fit the plan")
     _check(_fn("moe", "mi_moe_expert_gemm")(
         _p(x), _dt(x), ldx, x.shape[0], _p(weight), N * K, K, N, K, _p(plan.source), _p(plan.tile_expert),
-        plan.tile_expert.numel(), plan.pad, 1 if gather else 0, 1 if glu is not None else 0,
+        plan.tile_expert.numel(), plan.pad, 1 if gather else 0, 1 if glu is not None else (2 if squared_relu else 0),
         float(glu.limit) if glu is not None else 0.0, float(glu.alpha) if glu is not None else 0.0,
         float(glu.up_offset) if glu is not None else 0.0, _p(out), _dt(out), ldo, _stream()),
         "moe_expert_gemm", f"(N={N}, K={K})")
@@ -966,7 +1013,8 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                     tile_tokens: int = 0, cu_seqlens: Optional[torch.Tensor] = None,
                     log_bias: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
                     value_dim: Optional[int] = None, head_scales: Optional[torch.Tensor] = None,
-                    score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False) -> None:
+                    score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False, keep_first: int = 0,
+                    fixed_sink: Optional[float] = None) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
@@ -981,7 +1029,11 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     exp(sink) is one more term of the softmax's denominator, with no key and no value.  ``value_dim``: the
     width of a value head if it is not the keys'; ``out`` is then [T, Hq * value_dim].  ``head_scales`` (float32
     [Hq]): every head's scores are multiplied by its number (after ``scale``).  ``sigmoid``: a visible key weighs
-    sigmoid(score + ``score_bias[head]``) (float32 [Hq] or None) on its own and nothing is normalized."""
+    sigmoid(score + ``score_bias[head]``) (float32 [Hq] or None) on its own and nothing is normalized.
+    ``keep_first`` (with a window): keys at positions below it stay visible behind the window.  ``fixed_sink``: a
+    sink of this score for every head, in place of ``sinks``."""
+    _need(keep_first >= 0 and (keep_first == 0 or window), "paged_attention: first keys are kept behind a window")
+    _need(fixed_sink is None or (sinks is None and not sigmoid), "paged_attention: one sink, in a softmax")
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -1020,7 +1072,8 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     _check(_fn("attention", "mi_paged_attention")(
         _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, value_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
-        int(window or 0), _p(slopes), _p(log_bias), _p(sinks), span, _p(partial), partial.numel(), _p(out), out_ld,
+        int(window or 0), int(keep_first), _p(slopes), _p(log_bias), _p(sinks),
+        float(fixed_sink or 0.0), 0 if fixed_sink is None else 1, span, _p(partial), partial.numel(), _p(out), out_ld,
         _p(query_tiles) if tiles else None, tiles, int(tile_tokens) if tiles else 0, _p(cu_seqlens) if tiles else None,
         _p(head_scales), _p(score_bias), 1 if sigmoid else 0, _stream()), "paged_attention", f"(head_dim={head_dim})")
 
@@ -1030,14 +1083,21 @@ def attention_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head
                       slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                       v_cache: Optional[torch.Tensor], *, values_from_keys: bool = False,
                       q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
-                      norm_eps: float = 0.0, value_inv_freq: Optional[torch.Tensor] = None) -> None:
+                      norm_eps: float = 0.0, value_inv_freq: Optional[torch.Tensor] = None,
+                      interleaved: bool = False, turn_scale: float = 1.0, head_norm: Optional[str] = None,
+                      q_head_weight: Optional[torch.Tensor] = None, k_head_weight: Optional[torch.Tensor] = None,
+                      head_eps: float = 0.0) -> None:
     """A token's projected row made ready for attention, one launch: ``qkv`` [T, >= Hq*dh + Hkv*dh (+ Hkv*dv)]
     holds q heads, k heads and (unless ``values_from_keys``) v heads.
 
     * ``q_norm`` / ``k_norm`` (float32 [Hq*dh] / [Hkv*dh]): the whole q projection, and the whole k projection, is
       divided by its root mean square (``norm_eps`` inside the root) and multiplied by the weight, before rotation;
-    * q and k are turned by the token's position (half-split pairs over the first ``rotary_dim`` dims, angle =
-      position * inv_freq[j]); q is written back in place, k goes to the token's cache cell;
+    * ``head_norm`` ("before_rotation" / "after_rotation"): every q head and every k head is divided by its own root
+      mean square over dh (``head_eps`` inside the root) and multiplied by ``q_head_weight`` / ``k_head_weight``
+      (float32 [dh], shared by all heads; None: the bare division);
+    * q and k are turned by the token's position over the first ``rotary_dim`` dims, angle = position * inv_freq[j],
+      pairs (j, j + rotary_dim / 2) or, ``interleaved``, (2j, 2j + 1), cosines and sines times ``turn_scale``; q is
+      written back in place, k goes to the token's cache cell;
     * the values are the v heads, or with ``values_from_keys`` the k heads as projected (before norm and rotation);
       with ``value_inv_freq`` (float32 [dv / 2]) they are turned by the position over all their dims (half-split
       pairs); they go to the token's (transposed) cache cell.
@@ -1064,6 +1124,14 @@ def attention_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head
         _need(q_norm.dtype == torch.float32 and q_norm.numel() == q_cols and q_norm.is_contiguous() and q_norm.is_cuda
               and k_norm.dtype == torch.float32 and k_norm.numel() == k_cols and k_norm.is_contiguous()
               and k_norm.is_cuda and norm_eps > 0, "attention_prepare: the norms' weights must be float32 [Hq*dh], [Hkv*dh]")
+    _need(head_norm in (None, "before_rotation", "after_rotation") and (head_norm is None or q_norm is None),
+          "attention_prepare: heads are normed before or after the rotation, and not beside a norm of the projections")
+    _need((q_head_weight is None) == (k_head_weight is None) and (q_head_weight is None or head_norm is not None),
+          "attention_prepare: the heads' norm has both weights or none")
+    for one in (q_head_weight, k_head_weight):
+        _need(one is None or (one.dtype == torch.float32 and one.numel() == head_dim and one.is_contiguous() and one.is_cuda),
+              "attention_prepare: a weight of the heads' norm must be float32 [dh] on the GPU")
+    _need(head_norm is None or head_eps > 0, "attention_prepare: the heads' norm needs its eps")
     page_stride, page_size = 0, 0
     if slot_mapping is not None:
         _i32(slot_mapping, "slot_mapping")
@@ -1071,8 +1139,10 @@ def attention_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head
         page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, value_dim)
     _check(_fn("attention", "mi_attention_prepare")(
         _p(qkv), _dt(qkv), ld, T, num_heads, num_kv_heads, head_dim, value_dim, 1 if values_from_keys else 0,
-        _p(positions), _p(inv_freq), int(rotary_dim) if inv_freq is not None else 0, _p(q_norm), _p(k_norm),
-        float(norm_eps), _p(value_inv_freq), _p(slot_mapping), _p(k_cache) if slot_mapping is not None else None,
+        _p(positions), _p(inv_freq), int(rotary_dim) if inv_freq is not None else 0, 1 if interleaved else 0,
+        float(turn_scale), _p(q_norm), _p(k_norm), float(norm_eps),
+        {None: 0, "before_rotation": 1, "after_rotation": 2}[head_norm], _p(q_head_weight), _p(k_head_weight),
+        float(head_eps), _p(value_inv_freq), _p(slot_mapping), _p(k_cache) if slot_mapping is not None else None,
         _p(v_cache) if slot_mapping is not None else None, page_stride, page_size, _stream()), "attention_prepare")
 
 
@@ -1221,9 +1291,10 @@ def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
 # --------------------------------------------------------------------------- mamba2
 def conv1d_silu(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor,
                 bias: Optional[torch.Tensor], conv_state: torch.Tensor, lane_of_token: torch.Tensor,
-                cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor) -> None:
+                cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor, activation: bool = True) -> None:
     """out[t] = SiLU(causal depthwise conv of u[:, col_offset:col_offset+width]) per lane,
-    the K-1 rows before a lane's first token coming from ``conv_state[slot]`` [K-1, width]."""
+    the K-1 rows before a lane's first token coming from ``conv_state[slot]`` [K-1, width].
+    ``activation`` False: the convolution's sums as they are, without the SiLU."""
     ld = _row_major(u, "u")
     T = u.shape[0]
     K = weight.shape[1]
@@ -1238,7 +1309,7 @@ def conv1d_silu(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tens
         _i32(tensor, name)
     _check(_fn("mamba2", "mi_conv1d_silu")(
         _p(u), _dt(u), ld, col_offset, T, width, K, _p(weight), _p(bias), _p(conv_state), _p(lane_of_token),
-        _p(cu_seqlens), _p(slot_ids), _p(out), _stream()), "conv1d_silu", f"(K={K})")
+        _p(cu_seqlens), _p(slot_ids), _p(out), 1 if activation else 0, _stream()), "conv1d_silu", f"(K={K})")
 
 
 def conv_state_update(u: torch.Tensor, col_offset: int, width: int, kernel: int, conv_state: torch.Tensor,
@@ -1257,10 +1328,10 @@ def conv_state_update(u: torch.Tensor, col_offset: int, width: int, kernel: int,
 
 
 def conv_step(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
-              conv_state: torch.Tensor, slot_ids: torch.Tensor) -> None:
+              conv_state: torch.Tensor, slot_ids: torch.Tensor, activation: bool = True) -> None:
     """One conv step of single-token lanes, in place: row m of ``u`` is the new token of the request in
     ``slot_ids[m]``; columns [col_offset, col_offset + width) become SiLU(conv over [tail ; sample]) and the
-    tail ``conv_state[slot]`` [K-1, width] is rolled by one and takes the sample."""
+    tail ``conv_state[slot]`` [K-1, width] is rolled by one and takes the sample.  ``activation`` False: no SiLU."""
     ld = _row_major(u, "u")
     M = u.shape[0]
     K = weight.shape[1]
@@ -1273,7 +1344,8 @@ def conv_step(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor
     _i32(slot_ids, "slot_ids")
     _need(slot_ids.numel() >= M, "conv_step: one slot per row")
     _check(_fn("mamba2", "mi_conv_step")(_p(u), _dt(u), ld, col_offset, M, width, K, _p(weight), _p(bias),
-                                         _p(conv_state), _p(slot_ids), _stream()), "conv_step", f"(K={K})")
+                                         _p(conv_state), _p(slot_ids), 1 if activation else 0, _stream()),
+           "conv_step", f"(K={K})")
 
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,

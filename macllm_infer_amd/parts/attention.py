@@ -3,9 +3,9 @@ from __future__ import annotations
 
 import torch
 
-from ..cache.manager import KVNeed
+from ..cache.manager import KVNeed, StateNeed
 from ..kernels import ops
-from ..kernels.limits import ATTENTION_MAX_HEAD_DIM, GRID_MOST, beyond
+from ..kernels.limits import ATTENTION_MAX_HEAD_DIM, CONV_MAX_TAPS, GRID_MOST, beyond
 from ..weights.loader import Expect
 from .base import BuildContext, Mixer, part_class, register_part
 from .linear import Linear
@@ -27,14 +27,17 @@ class Attention(Mixer):
     Further forms, each a field of the spec: values that are the keys as projected (no v projection); an RMS norm
     over the whole q and the whole k projection before rotation; values turned by their position before they are
     cached and outputs turned back by the query's; a learned multiplier of every head's scores; sigmoid weights
-    with a learned bias per head in place of the softmax.  One kernel prepares a token's row for all of them
-    (``ops.attention_prepare``: norms, rotations, cache write).
+    with a learned bias per head in place of the softmax; an RMS norm of every q and k head, before or after the
+    rotation, with one weight for all heads or none; pairs of neighbouring dimensions turned, cosines and sines
+    times a magnitude; a window that keeps a sequence's first keys; a sink of a fixed score; a short causal
+    convolution over time behind the q, k and v projections, whose last rows are state of the request.  One kernel
+    prepares a token's row for all of them (``ops.attention_prepare``: norms, rotations, cache write).
 
     Multipliers: ``in_multiplier`` scales the input of q/k/v (folded into their weights),
     ``key_multiplier`` the k projection's output (weights and bias), ``out_multiplier``
     the output projection's output."""
     graph_safe = True
-    kernel_modules = ("common", "attention", "gemm")
+    kernel_modules = ("common", "attention", "gemm", "mamba2")
     query_tile = 64          # tokens of one lane that a workgroup of the prompt attention kernels takes
 
     @classmethod
@@ -59,6 +62,12 @@ class Attention(Mixer):
         if spec.projection_norm_eps is not None:
             out += [Expect(f"{prefix}.q_norm.weight", ((q_rows,),), init="norm"),
                     Expect(f"{prefix}.k_norm.weight", ((kv_rows,),), init="norm")]
+        if spec.head_norm is not None and spec.head_norm_weight:
+            out += [Expect(f"{prefix}.q_norm.weight", ((spec.head_dim,),), init="norm"),
+                    Expect(f"{prefix}.k_norm.weight", ((spec.head_dim,),), init="norm")]
+        if spec.conv_kernel > 0:
+            names = (("q_proj", q_rows), ("k_proj", kv_rows)) + (() if spec.values_from_keys else (("v_proj", v_rows),))
+            out += [Expect(f"{prefix}.{name}.conv.weight", ((rows, spec.conv_kernel),), init="conv") for name, rows in names]
         if spec.head_temperature:
             out.append(Expect(f"{prefix}.temp", ((spec.num_heads,),), init="positive"))
         if spec.score_bias:
@@ -71,12 +80,23 @@ class Attention(Mixer):
         return (beyond("attention", "head_dim", max(spec.head_dim, spec.value_width), ATTENTION_MAX_HEAD_DIM,
                        "a query row and its sums are kept in LDS and registers")
                 + beyond("attention", "num_heads", spec.num_heads, GRID_MOST, "heads index a dimension of the launch")
+                + beyond("attention", "conv_kernel", spec.conv_kernel, CONV_MAX_TAPS, "the taps of a channel are kept in registers")
                 + part_class(spec.position).limits(spec.position, spec.head_dim))
 
     @classmethod
+    def conv_width(cls, spec) -> int:
+        """The channels of the projections' convolution: q, k and v side by side."""
+        values = 0 if spec.values_from_keys else spec.num_kv_heads * spec.value_width
+        return (spec.num_heads + spec.num_kv_heads) * spec.head_dim + values
+
+    @classmethod
     def cache_needs(cls, spec):
-        return [KVNeed(spec.num_kv_heads, spec.head_dim, spec.window,
-                       None if spec.value_width == spec.head_dim else spec.value_width)]
+        needs = [KVNeed(spec.num_kv_heads, spec.head_dim, spec.window,
+                        None if spec.value_width == spec.head_dim else spec.value_width,
+                        spec.keep_first if spec.window else 0)]
+        if spec.conv_kernel > 1:       # the last taps - 1 projected rows of the request
+            needs.append(StateNeed("conv", (spec.conv_kernel - 1, cls.conv_width(spec)), "activation"))
+        return needs
 
     def __init__(self, spec, prefix: str, tensors, build: BuildContext):
         self.spec = spec
@@ -104,26 +124,38 @@ class Attention(Mixer):
             self.position = position_class(spec.position, spec.head_dim, build)
         f32 = lambda name: get(name).to(torch.float32).contiguous().to(build.device)
         self.sink = f32("sink") if spec.sink else None
+        self.fixed_sink = spec.fixed_sink
+        self.keep_first = int(spec.keep_first) if spec.window else 0
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))
         # the forms that ``ops.attention_prepare`` and the general kernel's extra terms serve
         self.head_scales = f32("temp") if spec.head_temperature else None
         self.score_bias = f32("pb") if spec.score_bias else None
         self.q_norm = f32("q_norm.weight") if spec.projection_norm_eps is not None else None
         self.k_norm = f32("k_norm.weight") if spec.projection_norm_eps is not None else None
+        weighted = spec.head_norm is not None and spec.head_norm_weight
+        self.q_head_weight = f32("q_norm.weight") if weighted else None
+        self.k_head_weight = f32("k_norm.weight") if weighted else None
+        self.conv_weight = None
+        if spec.conv_kernel > 0:       # the three convolutions as one over the columns [q | k | v], taps in float32
+            self.conv_weight = torch.cat([get(f"{name}.conv.weight").to(torch.float32).reshape(-1, spec.conv_kernel)
+                                          for name in names]).contiguous().to(build.device)
         self.value_inv_freq = None
         if spec.value_rotation_theta is not None:
             turns = rotary_frequencies(spec.value_rotation_theta, spec.value_width)
             self.value_inv_freq = torch.tensor(turns, dtype=torch.float64).to(torch.float32).to(build.device)
             self.value_inv_freq_back = (-self.value_inv_freq).contiguous()
+        pairs = self.position.pair_rotation()
         self.prepared = (spec.values_from_keys or spec.projection_norm_eps is not None
                          or spec.value_rotation_theta is not None or spec.head_temperature
-                         or spec.weighting != "softmax")
+                         or spec.weighting != "softmax" or spec.head_norm is not None or spec.conv_kernel > 0
+                         or self.fixed_sink is not None or self.keep_first > 0
+                         or (pairs is not None and (pairs[2] or self.position.magnitude != 1.0)))
+        self.interleaved = False
         if self.prepared:
-            rotation = self.position.fused_rotation()
-            if rotation is None or self.position.score_slopes is not None or self.position.score_log_bias is not None:
+            if pairs is None or self.position.score_slopes is not None or self.position.score_log_bias is not None:
                 raise ValueError(f"{prefix}: this form of attention turns q and k itself: the position encoding "
                                  f"{spec.position.kind!r} is no rotation by position")
-            self.inv_freq, self.rotary_dim = rotation
+            self.inv_freq, self.rotary_dim, self.interleaved = pairs
         # what only the general kernel knows: a bias on the scores, a sink, values of another width than the keys
         self.general_only = (self.position.score_slopes is not None or self.position.score_log_bias is not None
                              or self.sink is not None or spec.value_width != spec.head_dim or self.prepared)
@@ -202,11 +234,16 @@ class Attention(Mixer):
         spec = self.spec
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
         owns = cache.owns_kv
+        if self.conv_weight is not None:
+            qkv = self.convolve(qkv, step, cache)
         ops.attention_prepare(qkv, *geometry, spec.value_width, step.positions, self.inv_freq, self.rotary_dim,
                               step.slot_mappings[cache.group] if owns else None, cache.k_cache if owns else None,
                               cache.v_cache if owns else None, values_from_keys=spec.values_from_keys,
                               q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=spec.projection_norm_eps or 0.0,
-                              value_inv_freq=self.value_inv_freq)
+                              value_inv_freq=self.value_inv_freq, interleaved=self.interleaved,
+                              turn_scale=self.position.magnitude, head_norm=spec.head_norm,
+                              q_head_weight=self.q_head_weight, k_head_weight=self.k_head_weight,
+                              head_eps=spec.head_norm_eps if spec.head_norm is not None else 0.0)
         target = attended
         if self.value_inv_freq is not None:         # the heads' outputs are turned back into ``attended`` below
             target = torch.empty((qkv.shape[0], spec.num_heads * spec.value_width), dtype=qkv.dtype, device=qkv.device)
@@ -214,6 +251,22 @@ class Attention(Mixer):
         if target is not attended:
             ops.rotate_heads(target, 0, spec.value_width, spec.num_heads, spec.value_width, step.positions,
                              self.value_inv_freq_back, spec.value_width, False, attended, 0, spec.value_width)
+
+    def convolve(self, qkv: torch.Tensor, step, cache) -> torch.Tensor:
+        """The causal convolution over time of every column of the projected rows [q | k | v], the rows before a
+        lane's first token from the request's tail, which then takes the lane's last rows.  Single tokens: in
+        place, one launch."""
+        width, taps = self.conv_weight.shape
+        tail = cache.states["conv"] if taps > 1 else torch.empty((1, 0, width), dtype=qkv.dtype, device=qkv.device)
+        if step.max_query_len == 1:
+            ops.conv_step(qkv, 0, width, self.conv_weight, None, tail, step.slot_ids, activation=False)
+            return qkv
+        out = torch.empty((qkv.shape[0], width), dtype=qkv.dtype, device=qkv.device)
+        ops.conv1d_silu(qkv, 0, width, self.conv_weight, None, tail, step.lane_of_token, step.cu_seqlens, step.slot_ids,
+                        out, activation=False)
+        if taps > 1:
+            ops.conv_state_update(qkv, 0, width, taps, tail, step.cu_seqlens, step.slot_ids)
+        return out
 
     def attend_prepared(self, qkv: torch.Tensor, step, cache, out: torch.Tensor) -> None:
         spec = self.spec
@@ -223,6 +276,12 @@ class Attention(Mixer):
         if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
             tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
         plain = not sigmoid and self.head_scales is None and spec.value_width == spec.head_dim
+        if self.keep_first > 0 or self.fixed_sink is not None:
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, out, step.max_seq_len,
+                                value_dim=spec.value_width, head_scales=self.head_scales, keep_first=self.keep_first,
+                                fixed_sink=self.fixed_sink, **tiles)
+            return
         aligned = (qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 and out.stride(0) % 4 == 0
                    and out.data_ptr() % 8 == 0)
         if (step.max_query_len == 1 and aligned

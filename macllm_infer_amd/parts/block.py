@@ -69,7 +69,9 @@ class ParallelPreNormBlock:
     (reference: src/decoder.rs:2658-2682, 2684-2699).  With one mixer this is the ordinary
     sequential pre-norm layer.  A layer may scale either branch feature by feature before the add
     (``mixer_scale_name`` / ``ffn_scale_name``: h += scale * branch, the product in float32) or multiply both by
-    one number (``branch_multiplier``), and may have no feed-forward at all (``ffn`` None)."""
+    one number (``branch_multiplier``), and may have no feed-forward at all (``ffn`` None).  A mixer may have an RMS
+    norm of its own on its output (``MixerSlot.post_norm``): the normed outputs are summed with the mixers' weights
+    in one launch, in float32, and that sum is the branch."""
 
     @classmethod
     def expected_tensors(cls, layer, hidden_size: int):
@@ -78,6 +80,9 @@ class ParallelPreNormBlock:
             layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}", hidden_size)
         for slot in layer.mixers:
             out += part_class(slot.spec).expected_tensors(slot.spec, f"{layer.prefix}.{slot.name}", hidden_size)
+            if getattr(slot, "post_norm", None) is not None:
+                out += part_class(slot.post_norm).expected_tensors(
+                    slot.post_norm, f"{layer.prefix}.{slot.name}.{slot.post_norm_name}", hidden_size)
         if layer.mixer_scale_name:
             out.append(Expect(f"{layer.prefix}.{layer.mixer_scale_name}", ((hidden_size,),), init="scale"))
         second = part_class(layer.ffn_norm).expected_tensors(
@@ -133,7 +138,18 @@ class ParallelPreNormBlock:
         # the fast path knows plain branches and a feed-forward behind them; None when parts or sizes do not fit
         self.branch_multiplier = float(getattr(layer, "branch_multiplier", 1.0))
         self.mixer_weights = [float(getattr(slot, "weight", 1.0)) for slot in layer.mixers]
-        plain = (self.mixer_scale is None and self.ffn_scale is None and self.ffn is not None
+        # (weight, eps) of the RMS norm on a mixer's output, or None
+        self.mixer_posts = []
+        for slot in layer.mixers:
+            post = getattr(slot, "post_norm", None)
+            if post is None:
+                self.mixer_posts.append(None)
+                continue
+            if post.kind != "rmsnorm":
+                raise ValueError(f"layer {layer.prefix}: the norm on a mixer's output is an RMS norm")
+            norm = part_class(post)(post, f"{layer.prefix}.{slot.name}.{slot.post_norm_name}", tensors, build)
+            self.mixer_posts.append((norm.weight, float(post.eps)))
+        plain = (self.mixer_scale is None and all(post is None for post in self.mixer_posts) and self.ffn_scale is None and self.ffn is not None
                  and self.branch_multiplier == 1.0 and all(weight == 1.0 for weight in self.mixer_weights))
         self.fusion = factory(self, build) if factory is not None and plain else None
 
@@ -162,7 +178,9 @@ class ParallelPreNormBlock:
             return
         normed = self.mixer_norm.forward(residual)
         outputs = self.run_mixers(normed, step, caches)
-        if self.mixer_scale is not None:
+        if any(post is not None for post in self.mixer_posts):
+            outputs = self.normed_outputs(outputs)
+        elif self.mixer_scale is not None:
             outputs = [ScaledBranch(rows, self.mixer_scale) for rows in outputs]
         elif self.branch_multiplier != 1.0 or any(weight != 1.0 for weight in self.mixer_weights):
             outputs = [WeightedBranch(rows, self.branch_multiplier * weight)
@@ -178,6 +196,23 @@ class ParallelPreNormBlock:
             residual.pending = [WeightedBranch(rows, self.branch_multiplier)]
         else:
             residual.pending = [rows]
+
+    def normed_outputs(self, outputs: list) -> list:
+        """The mixers' outputs behind their own RMS norms: the normed ones summed with their weights in one launch
+        (float32), the others as weighted branches beside that sum."""
+        from ..kernels import ops
+        if self.mixer_scale is not None:
+            raise NotImplementedError("a scale by feature beside norms on the mixers' outputs")
+        normed = [(rows, weight, *post) for rows, weight, post in zip(outputs, self.mixer_weights, self.mixer_posts)
+                  if post is not None]
+        total = torch.empty(outputs[0].shape, dtype=torch.float32, device=outputs[0].device)
+        if len(normed) > ops.NORMED_SUM_MOST:
+            raise NotImplementedError(f"more than {ops.NORMED_SUM_MOST} mixers with norms on their outputs")
+        ops.normed_sum(normed, total)
+        branches = [WeightedBranch(total, self.branch_multiplier)]
+        branches += [WeightedBranch(rows, self.branch_multiplier * weight)
+                     for rows, weight, post in zip(outputs, self.mixer_weights, self.mixer_posts) if post is None]
+        return branches
 
     def run_mixers(self, normed: torch.Tensor, step, caches) -> list:
         """Every mixer's output for the normed rows, in the mixers' order."""

@@ -14,7 +14,7 @@ from .linear import Linear
 @register_part("latent_attention")
 class LatentAttention(Mixer):
     """Queries through a latent (c_q = RMSNorm(W_dq x), q = W_uq c_q: per head ``head_dim`` plain and ``rope_dim``
-    turned dimensions), keys and values through another (W_dkv x = [c before its RMSNorm | one turned key part for
+    turned dimensions) or, without a ``q_rank``, projected directly (q = W_q x); keys and values through another (W_dkv x = [c before its RMSNorm | one turned key part for
     all heads]; a head's plain key is W_uk c, its value W_uv c).
 
     The cache holds, per token, c and the turned key part: one "key" of ``kv_rank + rope_dim`` numbers shared by
@@ -33,9 +33,13 @@ class LatentAttention(Mixer):
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
         heads = spec.num_heads
-        return [Expect(f"{prefix}.dq.weight", ((spec.q_rank, hidden_size),)),
-                Expect(f"{prefix}.dq.norm.weight", ((spec.q_rank,),), init="norm"),
-                Expect(f"{prefix}.uq.weight", ((heads * (spec.head_dim + spec.rope_dim), spec.q_rank),)),
+        if spec.q_rank is None:
+            queries = [Expect(f"{prefix}.q.weight", ((heads * (spec.head_dim + spec.rope_dim), hidden_size),))]
+        else:
+            queries = [Expect(f"{prefix}.dq.weight", ((spec.q_rank, hidden_size),)),
+                       Expect(f"{prefix}.dq.norm.weight", ((spec.q_rank,),), init="norm"),
+                       Expect(f"{prefix}.uq.weight", ((heads * (spec.head_dim + spec.rope_dim), spec.q_rank),))]
+        return queries + [
                 Expect(f"{prefix}.dkv.weight", ((spec.kv_rank + spec.rope_dim, hidden_size),)),
                 Expect(f"{prefix}.dkv.norm.weight", ((spec.kv_rank,),), init="norm"),
                 Expect(f"{prefix}.uk.weight", ((heads * spec.head_dim, spec.kv_rank),)),
@@ -57,11 +61,18 @@ class LatentAttention(Mixer):
         self.build = build
         get = lambda name: tensors[f"{prefix}.{name}"]
         heads, dim, rope, rank = spec.num_heads, spec.head_dim, spec.rope_dim, spec.kv_rank
-        # both down-projections read the same rows: one product, [query latent | key/value latent | turned key part]
-        self.down = Linear([get("dq.weight"), get("dkv.weight")], [None, None], build)
-        self.up_q = Linear([get("uq.weight")], [None], build)
+        # both down-projections read the same rows: one product, [query latent | key/value latent | turned key part];
+        # without a query latent the queries themselves stand in its place
+        self.direct = spec.q_rank is None
+        self.q_width = heads * (dim + rope)
+        if self.direct:
+            self.down = Linear([get("q.weight"), get("dkv.weight")], [None, None], build)
+            self.up_q = self.q_norm = None
+        else:
+            self.down = Linear([get("dq.weight"), get("dkv.weight")], [None, None], build)
+            self.up_q = Linear([get("uq.weight")], [None], build)
+            self.q_norm = get("dq.norm.weight").to(torch.float32).contiguous().to(build.device)
         self.out = Linear([get("o.weight")], [None], build)
-        self.q_norm = get("dq.norm.weight").to(torch.float32).contiguous().to(build.device)
         self.kv_norm = get("dkv.norm.weight").to(torch.float32).contiguous().to(build.device)
         # per head: W_uk^T [kv_rank, head_dim] takes a plain query into the latent space; W_uv [value_dim, kv_rank]
         # takes an attended latent up.  Both are what the product of a head contracts over its rows with.
@@ -83,13 +94,18 @@ class LatentAttention(Mixer):
         heads, dim, rope, rank = spec.num_heads, spec.head_dim, spec.rope_dim, spec.kv_rank
         tokens = x.shape[0]
         down = self.down(x)
-        query_latent = torch.empty((tokens, spec.q_rank), dtype=x.dtype, device=x.device)
         owns = cache.owns_kv
-        ops.latent_prepare(down, spec.q_rank, rank, rope, self.q_norm, self.kv_norm, spec.norm_eps, step.positions,
-                           self.inv_freq, self.rotary_dim, self.interleaved,
-                           step.slot_mappings[cache.group] if owns else None, cache.k_cache if owns else None,
-                           cache.v_cache if owns else None, query_latent)
-        q = self.up_q(query_latent)                                   # [T, heads * (dim + rope)]
+        cells = (step.slot_mappings[cache.group] if owns else None, cache.k_cache if owns else None,
+                 cache.v_cache if owns else None)
+        if self.direct:
+            ops.latent_prepare(down[:, self.q_width:], 0, rank, rope, None, self.kv_norm, spec.norm_eps, step.positions,
+                               self.inv_freq, self.rotary_dim, self.interleaved, *cells, None)
+            q = down[:, :self.q_width]                                # [T, heads * (dim + rope)], a view
+        else:
+            query_latent = torch.empty((tokens, spec.q_rank), dtype=x.dtype, device=x.device)
+            ops.latent_prepare(down, spec.q_rank, rank, rope, self.q_norm, self.kv_norm, spec.norm_eps, step.positions,
+                               self.inv_freq, self.rotary_dim, self.interleaved, *cells, query_latent)
+            q = self.up_q(query_latent)                               # [T, heads * (dim + rope)]
         width = rank + rope
         latent_q = torch.empty((tokens, heads * width), dtype=x.dtype, device=x.device)
         ops.head_linear(q, 0, dim + rope, self.into_latent, latent_q, 0, width)

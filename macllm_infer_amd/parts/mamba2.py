@@ -42,7 +42,7 @@ class Mamba2(Mixer):
                     Expect(f"{prefix}.out_proj.bias", ((hidden_size,),), init="bias")]
         if spec.gated_norm:
             out.append(Expect(f"{prefix}.norm.weight",
-                              ((spec.num_groups, spec.inner_size // spec.num_groups), (spec.inner_size,)),
+                              ((spec.inner_size,), (spec.norm_parts, spec.inner_size // spec.norm_parts)),
                               init="norm"))
         return out
 
@@ -146,4 +146,4 @@ class Mamba2(Mixer):
             y = torch.empty((T, E), dtype=torch.float32, device=u.device)
             ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
                          step.slot_ids, spec.num_groups, y, step.max_query_len)
-        ops.gate_norm(y, u[:, :E], self.norm_weight, spec.num_groups, spec.norm_eps, gated)
+        ops.gate_norm(y, u[:, :E], self.norm_weight, spec.norm_parts, spec.norm_eps, gated)

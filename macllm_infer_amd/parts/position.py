@@ -34,6 +34,9 @@ class PositionEncoding(Part):
         layer then runs this part's own ``rotate_and_store`` and the general kernels."""
         return None
 
+    # what the cosines and sines of a rotation are multiplied by (a scaling of the frequencies may bring one)
+    magnitude = 1.0
+
     def pair_rotation(self):
         """``(inv_freq or None, rotary_dim, interleaved)`` of an encoding that turns pairs of dimensions by
         position * inv_freq[i]: pair i is dimensions (i, i + rotary_dim / 2) (half-split) or (2i, 2i + 1)
@@ -68,11 +71,24 @@ class NoPosition(PositionEncoding):
 def rotary_frequencies(theta: float, rotary_dim: int, scaling=None) -> list:
     """f_j = theta^(-2j / rotary_dim), j below rotary_dim / 2, in float64; with ``scaling`` (factor, low, high,
     original) stretched by wavelength l = 2 pi / f: kept where l < original / high, f / factor where
-    l > original / low, between the two (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    l > original / low, between the two (1 - s) f / factor + s f with s = (original / l - low) / (high - low).
+    A ``scaling`` with ``fast`` and ``slow`` (``RampScalingSpec``) blends f_j with f_j / factor by a ramp over j."""
     import math
     frequencies = [1.0 / (theta ** (index / rotary_dim)) for index in range(0, rotary_dim, 2)]
     if scaling is None:
         return frequencies
+    if hasattr(scaling, "fast"):
+        # blended by a ramp over the pair index: where(t) = dims ln(original / (2 pi t)) / (2 ln theta) is the index
+        # of the pair that makes t turns over the original context
+        def where(turns: float) -> float:
+            return rotary_dim * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+        low = max(math.floor(where(scaling.fast)), 0)
+        high = min(math.ceil(where(scaling.slow)), rotary_dim - 1)
+        out = []
+        for index, frequency in enumerate(frequencies):
+            ramp = min(max((index - low) / max(high - low, scaling.min_span), 0.0), 1.0)
+            out.append(frequency / scaling.factor * ramp + frequency * (1.0 - ramp))
+        return out
     out = []
     for frequency in frequencies:
         wavelength = 2.0 * math.pi / frequency
@@ -95,10 +111,14 @@ class Rope(PositionEncoding):
 
     def __init__(self, spec, head_dim: int, build: BuildContext):
         self.rotary_dim = spec.rotary_dim
-        frequencies = rotary_frequencies(spec.theta, spec.rotary_dim, getattr(spec, "scaling", None))
+        scaling = getattr(spec, "scaling", None)
+        frequencies = rotary_frequencies(spec.theta, spec.rotary_dim, scaling)
         self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+        self.magnitude = float(getattr(scaling, "magnitude", 1.0))
 
     def fused_rotation(self):
+        if self.magnitude != 1.0:          # the kernels that turn q and k themselves know no magnitude
+            return None
         return self.inv_freq, self.rotary_dim
 
     def pair_rotation(self):
@@ -141,8 +161,10 @@ class InterleavedRope(PositionEncoding):
 
     def __init__(self, spec, head_dim: int, build: BuildContext):
         self.rotary_dim = spec.rotary_dim
-        frequencies = [spec.theta ** (-index / spec.rotary_dim) for index in range(0, spec.rotary_dim, 2)]
+        scaling = getattr(spec, "scaling", None)
+        frequencies = rotary_frequencies(spec.theta, spec.rotary_dim, scaling)
         self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+        self.magnitude = float(getattr(scaling, "magnitude", 1.0))
 
     def pair_rotation(self):
         return self.inv_freq, self.rotary_dim, True

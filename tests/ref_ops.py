@@ -46,7 +46,8 @@ def cast_rows(source, out):
 
 def attention_prepare(qkv, num_heads, num_kv_heads, head_dim, value_dim, positions, inv_freq, rotary_dim, slot_mapping,
                       k_cache, v_cache, *, values_from_keys=False, q_norm=None, k_norm=None, norm_eps=0.0,
-                      value_inv_freq=None):
+                      value_inv_freq=None, interleaved=False, turn_scale=1.0, head_norm=None, q_head_weight=None,
+                      k_head_weight=None, head_eps=0.0):
     T = qkv.shape[0]
     q_cols, k_cols = num_heads * head_dim, num_kv_heads * head_dim
     q = _f(qkv[:, :q_cols]).clone()
@@ -62,14 +63,29 @@ def attention_prepare(qkv, num_heads, num_kv_heads, head_dim, value_dim, positio
     k = k.reshape(T, num_kv_heads, head_dim)
     spots = positions.to(torch.float32)
 
-    def rotate(x, frequencies, width):
+    def rotate(x, frequencies, width, neighbours=False, magnitude=1.0):
         half = width // 2
         angle = spots[:, None] * frequencies[None, :]
-        cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+        cos, sin = angle.cos()[:, None, :] * magnitude, angle.sin()[:, None, :] * magnitude
+        if neighbours:
+            out = x.clone()
+            a, b = x[..., 0:width:2], x[..., 1:width:2]
+            out[..., 0:width:2] = a * cos - b * sin
+            out[..., 1:width:2] = b * cos + a * sin
+            return out
         a, b = x[..., :half], x[..., half:width]
         return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., width:]], dim=-1)
+
+    def norm_heads(x, weight):
+        x = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + head_eps)
+        return x if weight is None else x * weight
+    if head_norm == "before_rotation":
+        q, k = norm_heads(q, q_head_weight), norm_heads(k, k_head_weight)
     if inv_freq is not None and rotary_dim > 0:
-        q, k = rotate(q, inv_freq, rotary_dim), rotate(k, inv_freq, rotary_dim)
+        q = rotate(q, inv_freq, rotary_dim, interleaved, turn_scale)
+        k = rotate(k, inv_freq, rotary_dim, interleaved, turn_scale)
+    if head_norm == "after_rotation":
+        q, k = norm_heads(q, q_head_weight), norm_heads(k, k_head_weight)
     if value_inv_freq is not None:
         v = rotate(v, value_inv_freq, value_dim)
     qkv[:, :q_cols] = q.reshape(T, q_cols).to(qkv.dtype)
@@ -160,7 +176,7 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
                     positions, scale, window, out, max_seq_len=None, slopes=None, query_tiles=None, tile_tokens=0,
                     cu_seqlens=None, log_bias=None, sinks=None, value_dim=None, head_scales=None, score_bias=None,
-                    sigmoid=False):
+                    sigmoid=False, keep_first=0, fixed_sink=None):
     """``max_seq_len`` sizes the kernel's launch and nothing else: not used here, and neither is the table of
     runs that picks the kernel for lanes of several tokens.  ``slopes``: a bias on the scores,
     ``-slopes[head] * (query position - key position)``; ``log_bias`` [Hq, 2] = (r1, r2): the scores lose
@@ -174,6 +190,8 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
         position = int(positions[token])
         first = 0 if not window else max(0, position - window + 1)
         keys = torch.arange(first, position + 1)
+        if keep_first and first > 0:
+            keys = torch.cat([torch.arange(0, min(keep_first, first)), keys])
         pages = block_tables[lane][(keys // page_size).long()].long()
         offsets = (keys % page_size).long()
         k = _f(k_cache[pages, :, offsets, :])        # [keys, Hkv, dh]
@@ -191,7 +209,9 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
                 scores = scores - slopes[head] * (position - keys).float()
             if log_bias is not None:
                 scores = scores - log_bias[head, 0] * torch.log1p(log_bias[head, 1] * (position - keys).float())
-            if sinks is not None:
+            if fixed_sink is not None:
+                weights = torch.softmax(torch.cat([scores, torch.tensor([float(fixed_sink)])]), dim=0)[:-1]
+            elif sinks is not None:
                 weights = torch.softmax(torch.cat([scores, sinks[head].reshape(1)]), dim=0)[:-1]
             else:
                 weights = torch.softmax(scores, dim=0)
@@ -213,7 +233,7 @@ def decode_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, blo
                     sigmoid=sigmoid)
 
 
-def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out):
+def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out, activation=True):
     K = weight.shape[1]
     for lane in range(slot_ids.numel()):
         begin, end = int(cu_seqlens[lane]), int(cu_seqlens[lane + 1])
@@ -224,7 +244,7 @@ def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, c
             total += window[tap:tap + end - begin] * weight[:, tap][None, :]
         if bias is not None:
             total += bias[None, :]
-        out[begin:end] = F.silu(total).to(out.dtype)
+        out[begin:end] = (F.silu(total) if activation else total).to(out.dtype)
 
 
 def conv_state_update(u, col_offset, width, kernel, conv_state, cu_seqlens, slot_ids):
@@ -237,11 +257,11 @@ def conv_state_update(u, col_offset, width, kernel, conv_state, cu_seqlens, slot
         conv_state[slot] = window[-(kernel - 1):]
 
 
-def conv_step(u, col_offset, width, weight, bias, conv_state, slot_ids):
+def conv_step(u, col_offset, width, weight, bias, conv_state, slot_ids, activation=True):
     M = u.shape[0]
     lanes = torch.arange(M + 1, dtype=torch.int32)
     out = torch.empty((M, width), dtype=u.dtype)
-    conv1d_silu(u, col_offset, width, weight, bias, conv_state, lanes[:M], lanes, slot_ids[:M], out)
+    conv1d_silu(u, col_offset, width, weight, bias, conv_state, lanes[:M], lanes, slot_ids[:M], out, activation)
     conv_state_update(u, col_offset, width, weight.shape[1], conv_state, lanes, slot_ids[:M])
     u[:, col_offset:col_offset + width] = out
 
@@ -446,7 +466,8 @@ def latent_prepare(down, q_rank, kv_rank, rope_dim, q_norm, kv_norm, eps, positi
     rows = _f(down)
     def rms(x, weight):
         return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * weight
-    query_latent.copy_(rms(rows[:, :q_rank], q_norm).to(query_latent.dtype))
+    if q_rank > 0:
+        query_latent.copy_(rms(rows[:, :q_rank], q_norm).to(query_latent.dtype))
     if slot_mapping is None:
         return
     latent = rms(rows[:, q_rank:q_rank + kv_rank], kv_norm)
@@ -479,7 +500,12 @@ def latent_attention_supported(dtype, num_heads, kv_rank, rope_dim, page_size):
 
 
 # --------------------------------------------------------------------------- routed experts
-def moe_route(logits, num_experts, top_k, correction, scale, eps, shared_gate):
+def moe_route(logits, num_experts, top_k, correction, scale, eps, shared_gate, routing="softmax_then_top"):
+    if routing == "top_then_softmax":
+        biased = _f(logits[:, :num_experts]) + correction
+        picked, chosen = torch.topk(biased, top_k, dim=-1)
+        gate = torch.sigmoid(_f(logits[:, num_experts])) if shared_gate else None
+        return chosen.to(torch.int32), torch.softmax(picked, dim=-1) * scale, gate
     scores = torch.softmax(_f(logits[:, :num_experts]), dim=-1)
     chosen = torch.topk(scores + correction, top_k, dim=-1).indices
     picked = torch.gather(scores, 1, chosen)
@@ -512,7 +538,7 @@ def moe_plan(chosen, num_experts, pad=None):
     return MoePlan(chosen, num_experts, pad or 16)
 
 
-def moe_expert_gemm(x, plan, weight, out, gather, glu):
+def moe_expert_gemm(x, plan, weight, out, gather, glu, squared_relu=False):
     out.zero_()
     for tile in range(plan.tile_expert.numel()):
         expert = int(plan.tile_expert[tile])
@@ -529,7 +555,17 @@ def moe_expert_gemm(x, plan, weight, out, gather, glu):
                 gate = sums[:inner].clamp(max=glu.limit)
                 up = sums[inner:].clamp(min=-glu.limit, max=glu.limit)
                 sums = gate * torch.sigmoid(glu.alpha * gate) * (up + glu.up_offset)
+            elif squared_relu:
+                sums = torch.relu(sums) ** 2
             out[place] = sums.to(out.dtype)
+
+
+def normed_sum(branches, out):
+    total = torch.zeros(out.shape, dtype=torch.float32)
+    for rows, factor, weight, eps in branches:
+        x = _f(rows)
+        total += factor * (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight)
+    out.copy_(total)
 
 
 def moe_combine(down, plan, weights, shared_rows, shared_gate, out):
@@ -545,7 +581,7 @@ NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supporte
          "add_scaled_rmsnorm", "polynorm", "tanh_rows", "head_norm_gate", "linear_state_scan",
          "embed_bigram", "stream_add", "add_layernorm", "clamped_glu", "latent_prepare", "head_linear", "rotate_heads",
          "latent_attention_supported", "moe_route", "moe_plan", "moe_expert_gemm", "moe_combine", "cast_rows",
-         "attention_prepare"]
+         "attention_prepare", "normed_sum"]
 
 
 def install(monkeypatch):
