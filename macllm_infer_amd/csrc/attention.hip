@@ -892,6 +892,9 @@ struct alignas(16) bf16x8 {
 // (a multiplier on a head's scores, after `scale`) and score_bias may be null.  sigmoid: a visible key weighs
 // sigmoid(score + score_bias[head]) on its own; the block then records (0, 1) as its (max, sum) and the merge adds
 // the partial outputs as they are.  Dynamic LDS: DEC_WAVES * G * dv floats.
+// kept > 0 (with a window): the keys at positions below kept stay visible; those that lie before the window's first
+// page are the work of one more block, blockIdx.x == splits, whose partial result stands behind the others'
+// (an empty one, maximum -inf, when the window still reaches them).
 template <int DH, int G>
 __global__ void __launch_bounds__(DEC_THREADS)
 decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const bf16_t* __restrict__ k_base,
@@ -900,7 +903,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
                         const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
                         int window, int split_keys, int splits, float* __restrict__ partial_o,
                         float* __restrict__ partial_ml, int dv, const float* __restrict__ head_scales,
-                        const float* __restrict__ score_bias, int sigmoid) {
+                        const float* __restrict__ score_bias, int sigmoid, int kept) {
   constexpr int LPR = DH / 8;
   constexpr int KPW = WAVE / LPR;
   constexpr int KPB = KPW * DEC_WAVES;
@@ -914,12 +917,25 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
   const int pos = positions[token];
   int first_key = 0;
   if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
-  const int range_lo = (first_key / page_size) * page_size + split * split_keys;
+  const int first_page_key = (first_key / page_size) * page_size;
+  const bool kept_block = split == splits;                   // only launched with kept > 0
+  const int stride = kept > 0 ? splits + 1 : splits;         // partial results of a head
+  const int range_lo = kept_block ? 0 : first_page_key + split * split_keys;
   if (range_lo > pos) return;
-  const int range_hi = min(range_lo + split_keys, pos + 1);
+  const int range_hi = kept_block ? min(kept, first_page_key) : min(range_lo + split_keys, pos + 1);
   const int count = range_hi - range_lo;
-  const int* table = block_tables + (long)lane_of_token[token] * max_pages;
   const int tid = threadIdx.x;
+  if (count <= 0) {          // the kept first keys are inside the window's pages: nothing of their own
+    for (int index = tid; index < G * dv; index += DEC_THREADS)
+      partial_o[((token * Hq + kvh * G + index / dv) * stride + split) * dv + index % dv] = 0.f;
+    if (tid < G) {
+      float* ml = partial_ml + ((token * Hq + kvh * G + tid) * stride + split) * 2;
+      ml[0] = sigmoid ? 0.f : -INFINITY;
+      ml[1] = sigmoid ? 1.f : 0.f;
+    }
+    return;
+  }
+  const int* table = block_tables + (long)lane_of_token[token] * max_pages;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
   const int r = lane / LPR;
@@ -963,7 +979,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
       for (int g = 0; g < G; ++g) s[g] += __shfl_xor(s[g], offset, WAVE);
     if (valid && c == 0) {
 #pragma unroll
-      for (int g = 0; g < G; ++g) s_lds[g][local] = key >= first_key ? s[g] + offset_of[g] : -INFINITY;
+      for (int g = 0; g < G; ++g) s_lds[g][local] = (key >= first_key || key < kept) ? s[g] + offset_of[g] : -INFINITY;
     }
   }
   __syncthreads();
@@ -1002,7 +1018,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
     for (int g = 0; g < G; ++g) {
       float sum = 0.f;
       for (int i = tid; i < count; i += DEC_THREADS) {
-        const float p = __expf(s_lds[g][i] - m[g]);
+        const float p = m[g] == -INFINITY ? 0.f : __expf(s_lds[g][i] - m[g]);
         s_lds[g][i] = p;
         sum += p;
       }
@@ -1056,10 +1072,10 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) sum += acc_lds[((long)w * G + g) * dv + dim];
-    partial_o[((token * Hq + kvh * G + g) * splits + split) * dv + dim] = sum;
+    partial_o[((token * Hq + kvh * G + g) * stride + split) * dv + dim] = sum;
   }
   if (tid < G) {
-    float* ml = partial_ml + ((token * Hq + kvh * G + tid) * splits + split) * 2;
+    float* ml = partial_ml + ((token * Hq + kvh * G + tid) * stride + split) * 2;
     ml[0] = m[tid];
     ml[1] = l[tid];
   }
@@ -1070,7 +1086,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const b
 __global__ void decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
                                     const int* __restrict__ positions, int window, int page_size,
                                     int split_keys, int splits, int Hq, int dh, bf16_t* __restrict__ out,
-                                    long out_ld, int sigmoid) {
+                                    long out_ld, int sigmoid, int kept, const float* __restrict__ sinks) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int pos = positions[token];
@@ -1078,13 +1094,33 @@ __global__ void decode_merge_kernel(const float* __restrict__ partial_o, const f
   if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
   const int first_page_key = (first_key / page_size) * page_size;
   const int used = min(splits, (pos - first_page_key) / split_keys + 1);
-  const float* ml = partial_ml + (token * Hq + head) * splits * 2;
-  const float* o = partial_o + (token * Hq + head) * (long)splits * dh;
+  const int stride = kept > 0 ? splits + 1 : splits;
+  const float* ml = partial_ml + (token * Hq + head) * stride * 2;
+  const float* o = partial_o + (token * Hq + head) * (long)stride * dh;
   if (sigmoid) {
     for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
       float sum = 0.f;
       for (int s = 0; s < used; ++s) sum += o[(long)s * dh + dim];
+      if (kept > 0) sum += o[(long)splits * dh + dim];
       out[token * out_ld + (long)head * dh + dim] = (bf16_t)sum;
+    }
+    return;
+  }
+  if (kept > 0 || sinks) {
+    // the block of the kept first keys and a sink (a term of the denominator that brings no value) beside the splits
+    const float sink = sinks ? sinks[head] : -INFINITY;
+    float maximum = sink;
+    for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
+    if (kept > 0) maximum = fmaxf(maximum, ml[2 * splits]);
+    float denominator = sinks ? __expf(sink - maximum) : 0.f;
+    for (int s = 0; s < used; ++s) denominator += __expf(ml[2 * s] - maximum) * ml[2 * s + 1];
+    const float kept_factor = kept > 0 ? __expf(ml[2 * splits] - maximum) : 0.f;
+    if (kept > 0) denominator += kept_factor * ml[2 * splits + 1];
+    for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+      float sum = 0.f;
+      for (int s = 0; s < used; ++s) sum += __expf(ml[2 * s] - maximum) * o[(long)s * dh + dim];
+      if (kept > 0) sum += kept_factor * o[(long)splits * dh + dim];
+      out[token * out_ld + (long)head * dh + dim] = (bf16_t)(sum / denominator);
     }
     return;
   }
@@ -1131,28 +1167,32 @@ static int launch_decode(const bf16_t* q, long q_ld, int T, int Hq, int Hkv, con
                          const bf16_t* v_base, long page_stride, int page_size, const int* block_tables,
                          int max_pages, const int* lane_of_token, const int* positions, float scale, int window,
                          int split_keys, int splits, float* partial_o, float* partial_ml, int dv,
-                         const float* head_scales, const float* score_bias, int sigmoid, hipStream_t stream) {
-  const dim3 grid(splits, Hkv, T);
+                         const float* head_scales, const float* score_bias, int sigmoid, int kept, hipStream_t stream) {
+  const dim3 grid(kept > 0 ? splits + 1 : splits, Hkv, T);
   const size_t dynamic = sizeof(float) * DEC_WAVES * G * (size_t)dv;
   decode_attention_kernel<DH, G><<<grid, DEC_THREADS, dynamic, stream>>>(
       q, q_ld, Hq, k_base, v_base, page_stride, page_size, block_tables, max_pages, lane_of_token, positions,
-      scale, window, split_keys, splits, partial_o, partial_ml, dv, head_scales, score_bias, sigmoid);
+      scale, window, split_keys, splits, partial_o, partial_ml, dv, head_scales, score_bias, sigmoid, kept);
   return 0;
 }
 
 // Returns ERR_UNSUPPORTED_SIZE for shapes this kernel does not cover (the caller then uses
 // mi_paged_attention): head_dim 64 or 128, 1..8 query heads per kv head, page_size a multiple of 8,
 // split_keys a multiple of page_size and at most DEC_MAX_SPLIT, values of up to 256 dims a head.
-// partial_o holds T * Hq * splits * dv floats.
+// partial_o holds T * Hq * splits * dv floats (with kept > 0: splits + 1 a head, and partial_ml likewise).
+// kept (with a window): the first keys that stay visible, at most DEC_MAX_SPLIT; sinks (float32 per query head, or
+// null): exp(sink) is one more term of the softmax's denominator.
 extern "C" int mi_decode_attention_forms(const void* q, long q_ld, int T, int Hq, int Hkv, int dh, int dv,
                                          const void* k_base, const void* v_base, long page_stride, int page_size,
                                          const int* block_tables, int max_pages, const int* lane_of_token,
                                          const int* positions, float scale, int window, int split_keys, int splits,
                                          float* partial_o, float* partial_ml, void* out, long out_ld,
                                          const float* head_scales, const float* score_bias, int sigmoid,
-                                         hipStream_t stream) {
+                                         int kept, const float* sinks, hipStream_t stream) {
   if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || splits <= 0 || max_pages <= 0 || dv <= 0)
     return ERR_BAD_ARGUMENT;
+  if (kept < 0 || (kept > 0 && window <= 0) || (sinks && sigmoid)) return ERR_BAD_ARGUMENT;
+  if (kept > DEC_MAX_SPLIT) return ERR_UNSUPPORTED_SIZE;
   const int G = Hq / Hkv;
   if ((dh != 64 && dh != 128) || G > 8 || page_size % 8 != 0 || split_keys % page_size != 0 ||
       split_keys <= 0 || split_keys > DEC_MAX_SPLIT || T > 65535 || Hkv > 65535 || dv > 256)
@@ -1163,7 +1203,7 @@ extern "C" int mi_decode_attention_forms(const void* q, long q_ld, int T, int Hq
     launch_decode<DH_, G_>((const bf16_t*)q, q_ld, T, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base,     \
                            page_stride, page_size, block_tables, max_pages, lane_of_token, positions, scale,     \
                            window, split_keys, splits, partial_o, partial_ml, dv, head_scales, score_bias,       \
-                           sigmoid, stream);
+                           sigmoid, kept, stream);
   DECODE_CASE(64, 1) DECODE_CASE(64, 2) DECODE_CASE(64, 3) DECODE_CASE(64, 4) DECODE_CASE(64, 5)
   DECODE_CASE(64, 6) DECODE_CASE(64, 7) DECODE_CASE(64, 8)
   DECODE_CASE(128, 1) DECODE_CASE(128, 2) DECODE_CASE(128, 3) DECODE_CASE(128, 4) DECODE_CASE(128, 5)
@@ -1174,7 +1214,7 @@ extern "C" int mi_decode_attention_forms(const void* q, long q_ld, int T, int Hq
   const int merge_threads = dv <= 64 ? 64 : dv <= 128 ? 128 : 256;
   decode_merge_kernel<<<merge_grid, merge_threads, 0, stream>>>(partial_o, partial_ml, positions, window, page_size,
                                                                 split_keys, splits, Hq, dv, (bf16_t*)out, out_ld,
-                                                                sigmoid);
+                                                                sigmoid, kept, sinks);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -1187,7 +1227,7 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
                                    void* out, long out_ld, hipStream_t stream) {
   return mi_decode_attention_forms(q, q_ld, T, Hq, Hkv, dh, dh, k_base, v_base, page_stride, page_size, block_tables,
                                    max_pages, lane_of_token, positions, scale, window, split_keys, splits, partial_o,
-                                   partial_ml, out, out_ld, nullptr, nullptr, 0, stream);
+                                   partial_ml, out, out_ld, nullptr, nullptr, 0, 0, nullptr, stream);
 }
 
 // ---------------------------------------------------------------- decode attention without a workspace argument
@@ -1273,7 +1313,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
                          int window, bf16_t* __restrict__ out, long out_ld,
                          const float* __restrict__ log_bias = nullptr, const float* __restrict__ sinks = nullptr,
                          int value_dim = DV, const float* __restrict__ head_scales = nullptr,
-                         const float* __restrict__ score_bias = nullptr) {
+                         const float* __restrict__ score_bias = nullptr, int kept = 0) {
   constexpr int ITEMS = 2 + 4 * (DV / 16);                    // m, l and the accumulator of one set
   __shared__ float part[PREFILL_WAVES][ITEMS][WAVE];
   __shared__ int wave_pages[PREFILL_WAVES][WAVE];
@@ -1357,17 +1397,22 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   const int my_hi = min(key_hi, my_lo + 32 * steps_per_wave);
   // the page ids of the run go through LDS, 64 pages at a time (a wave's own corner of it: no
   // barrier), so that a K or V load does not wait for a load of its page id
-  for (int part_lo = my_lo; part_lo < my_hi;) {
-    const int first_page = part_lo / page_size;
-    const int part_hi = min(my_hi, (first_page + WAVE) * page_size);
-    wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
-    cache.pages = wave_pages[wave];
-    cache.base_page = first_page;
-    attend_keys<DH, NSET, PREFILL_STEPS, false, EXTRAS, DV, SIGMOID, PADDED>(
-        acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache, full_tile ? first_position : -1, last_position,
-        bias, &gate);
-    part_lo = part_hi;
-  }
+  auto walk = [&](int from, int to) {
+    for (int part_lo = from; part_lo < to;) {
+      const int first_page = part_lo / page_size;
+      const int part_hi = min(to, (first_page + WAVE) * page_size);
+      wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
+      cache.pages = wave_pages[wave];
+      cache.base_page = first_page;
+      attend_keys<DH, NSET, PREFILL_STEPS, false, EXTRAS, DV, SIGMOID, PADDED>(
+          acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache, full_tile ? first_position : -1, last_position,
+          bias, &gate, kept);
+      part_lo = part_hi;
+    }
+  };
+  walk(my_lo, my_hi);
+  // the kept first keys that lie before the window's first step: the last wave, whose own run is the shortest
+  if (kept > 0 && key_lo > 0 && wave == PREFILL_WAVES - 1) walk(0, min(kept, key_lo));
 
   // merge: set s is finished by wave s
 #pragma unroll
@@ -1499,9 +1544,11 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
                                     const void* v_base, long page_stride, int page_size, const int* block_tables,
                                     int max_pages, const int* tiles, int n_tiles, const int* cu_seqlens,
                                     const int* start_pos, float scale, int window, int max_seq_len, void* out,
-                                    long out_ld, const float* log_bias, const float* sinks, hipStream_t stream) {
+                                    long out_ld, const float* log_bias, const float* sinks, int kept,
+                                    hipStream_t stream) {
   if (n_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || max_pages <= 0)
     return ERR_BAD_ARGUMENT;
+  if (kept < 0 || (kept > 0 && window <= 0)) return ERR_BAD_ARGUMENT;      // first keys are kept behind a window
   const int G = Hq / Hkv;
   if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64)
     return ERR_UNSUPPORTED_SIZE;
@@ -1524,11 +1571,13 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
     if (extras)                                                                                               \
       prefill_attention_kernel<DH_, NSET_, true><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                  \
           (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
-          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, log_bias, sinks); \
+          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, log_bias, sinks, \
+          DH_, nullptr, nullptr, kept);                                                                       \
     else                                                                                                      \
       prefill_attention_kernel<DH_, NSET_><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                        \
           (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
-          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld);         \
+          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, nullptr, \
+          nullptr, DH_, nullptr, nullptr, kept);                                                              \
   }
   PREFILL_CASE(64, 1) PREFILL_CASE(64, 2) PREFILL_CASE(64, 3) PREFILL_CASE(64, 4)
   PREFILL_CASE(128, 1) PREFILL_CASE(128, 2) PREFILL_CASE(128, 3) PREFILL_CASE(128, 4)

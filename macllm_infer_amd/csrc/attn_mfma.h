@@ -15,7 +15,8 @@
 //            softmax (4 keys of tile 0, 4 keys of tile 1) are exactly its B fragment once the
 //            32 keys of the step are numbered (q, j) -> j < 4 ? 4q + j : 16 + 4q + (j - 4).
 // Formulas: s = q.k * scale, key visible when key <= column position and, with a window w,
-// position - key < w (reference: src/decoder.rs:4515-4532, 4641-4670); softmax in float32.
+// position - key < w (reference: src/decoder.rs:4515-4532, 4641-4670) or, with kept > 0, key < kept (the first
+// keys of a sequence stay visible behind the window); softmax in float32.
 #pragma once
 #include "common.h"
 
@@ -131,7 +132,7 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
                                              const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                              const int (&col_pos)[NSET], int window, float scale, int k00,
                                              int key_hi, const AttnLogBias<NSET>& bias = AttnLogBias<NSET>(),
-                                             const AttnGate<NSET>* gate = nullptr) {
+                                             const AttnGate<NSET>* gate = nullptr, int kept = 0) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int q = lane / 16;
   const int last_key = key_hi - 1;
@@ -189,11 +190,13 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
         const bool any = last_visible >= first_visible;
         const int lo = any ? first_visible - k0 : 0x40000000;
         const unsigned span = any ? (unsigned)(last_visible - first_visible) : 0u;
+        // the kept first keys of the column, relative to the step: offsets below kept_end (none: a negative end)
+        const int kept_end = min(kept, last_visible + 1) - k0;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const bool visible = (unsigned)(16 * t + 4 * q + i - lo) <= span;
+            const bool visible = (unsigned)(16 * t + 4 * q + i - lo) <= span || 16 * t + 4 * q + i < kept_end;
             score[t][i] = visible ? score[t][i] : -INFINITY;
           }
       }
@@ -263,7 +266,7 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET, DV>& acc,
                                             const int (&col_pos)[NSET], int window, float scale, int key_lo,
                                             int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1,
                                             const AttnLogBias<NSET>& bias = AttnLogBias<NSET>(),
-                                            const AttnGate<NSET>* gate = nullptr) {
+                                            const AttnGate<NSET>* gate = nullptr, int kept = 0) {
   const int last_key = key_hi - 1;
   constexpr int ROUND = 32 * STEPS;
   if (PIPELINED) {
@@ -294,7 +297,7 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET, DV>& acc,
       AttnFragments<DH, STEPS, DV> f;
       attn_load<DH, STEPS, DV, PADDED>(f, k00, last_key, cache);
       attn_compute<DH, NSET, STEPS, true, BIASED, DV, SIGMOID>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias,
-                                                               gate);
+                                                               gate, kept);
     }
   }
 }

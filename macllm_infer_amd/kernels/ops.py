@@ -105,7 +105,7 @@ _SIGNATURES = {
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
-                                 _c_ptr, _c_ptr, _c_ptr],
+                                 _c_ptr, _c_ptr, _c_int, _c_ptr],
         "mi_prefill_attention_forms": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                        _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr,
                                        _c_long, _c_int, _c_ptr, _c_ptr, _c_ptr],
@@ -114,7 +114,7 @@ _SIGNATURES = {
                                 _c_ptr, _c_long, _c_ptr],
         "mi_decode_attention_forms": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
                                       _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr,
-                                      _c_ptr, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_ptr],
+                                      _c_ptr, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
     },
     "mamba2": {
         "mi_conv1d_silu": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -1156,12 +1156,13 @@ def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                       v_cache: torch.Tensor, block_tables: torch.Tensor, query_tiles: torch.Tensor,
                       cu_seqlens: torch.Tensor, start_pos: torch.Tensor, scale: float, window: Optional[int],
                       out: torch.Tensor, max_seq_len: int = 0, log_bias: Optional[torch.Tensor] = None,
-                      sinks: Optional[torch.Tensor] = None) -> None:
+                      sinks: Optional[torch.Tensor] = None, keep_first: int = 0) -> None:
     """``paged_attention`` on the matrix cores for bfloat16 (flash-style, online softmax in
     float32).  ``query_tiles`` [tiles, 2]: (lane, first token row) of runs of up to 64 tokens of
     one lane; the keys and values of the step's own tokens must be in the cache already.
     ``max_seq_len``: an upper bound of the step's longest context if known (it picks how many heads share
-    a key fragment, never the result)."""
+    a key fragment, never the result).  ``keep_first`` (with a window): keys at positions below it stay visible."""
+    _need(keep_first >= 0 and (keep_first == 0 or window), "prefill_attention: first keys are kept behind a window")
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -1187,7 +1188,7 @@ def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         _p(q), q_ld, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
         _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
         _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, _p(log_bias),
-        _p(sinks), _stream()), "prefill_attention")
+        _p(sinks), int(keep_first), _stream()), "prefill_attention")
 
 
 PREFILL_VALUE_WIDTH_MOST = 256      # the widest values the matrix-core kernel computes with
@@ -1238,22 +1239,30 @@ def prefill_attention_forms(q: torch.Tensor, num_heads: int, num_kv_heads: int, 
         _p(head_scales), _p(score_bias), _stream()), "prefill_attention_forms")
 
 
+DECODE_KEEP_FIRST_MOST = 512        # DEC_MAX_SPLIT in attention.hip: the kept first keys are one block's work
+
+
 def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
-                               value_dim: Optional[int] = None) -> bool:
+                               value_dim: Optional[int] = None, keep_first: int = 0) -> bool:
     """Whether the split-context kernel for single-token queries covers this geometry."""
     return (dtype == torch.bfloat16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 8
-            and page_size % 8 == 0 and page_size <= 512 and (value_dim is None or 0 < value_dim <= 256))
+            and page_size % 8 == 0 and page_size <= 512 and (value_dim is None or 0 < value_dim <= 256)
+            and keep_first <= DECODE_KEEP_FIRST_MOST)
 
 
 def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, block_tables: torch.Tensor, lane_of_token: torch.Tensor,
                      positions: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
                      out: torch.Tensor, value_dim: Optional[int] = None, head_scales: Optional[torch.Tensor] = None,
-                     score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False) -> None:
+                     score_bias: Optional[torch.Tensor] = None, sigmoid: bool = False, keep_first: int = 0,
+                     sinks: Optional[torch.Tensor] = None) -> None:
     """``paged_attention`` for batches of single decoded tokens in bfloat16: the context of each
     request is split over many workgroups and the G query heads of a kv head share its K/V
     loads.  ``max_seq_len``: an upper bound of the longest context in the batch.  ``value_dim``,
-    ``head_scales``, ``score_bias`` and ``sigmoid`` as in ``paged_attention``."""
+    ``head_scales``, ``score_bias``, ``sigmoid``, ``keep_first`` and ``sinks`` as in ``paged_attention``."""
+    _need(keep_first >= 0 and (keep_first == 0 or window), "decode_attention: first keys are kept behind a window")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads and sinks.is_contiguous()
+                            and sinks.is_cuda and not sigmoid), "decode_attention: sinks must be float32 [Hq] on the GPU")
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -1262,7 +1271,7 @@ def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * value_dim) and q_ld % 8 == 0
           and q.data_ptr() % 16 == 0, "decode_attention: q/out shapes or alignment do not fit")
     page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype, value_dim)
-    _need(decode_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim),
+    _need(decode_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim, keep_first),
           "decode_attention: geometry not covered; use paged_attention")
     _i32(block_tables, "block_tables")
     _i32(lane_of_token, "lane_of_token")
@@ -1279,13 +1288,14 @@ def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         split_keys *= 2
     split_keys = max(split_keys, page_size)
     splits = max(1, -(-span // split_keys))
-    partial_o = torch.empty((T, num_heads, splits, value_dim), dtype=torch.float32, device=q.device)
-    partial_ml = torch.empty((T, num_heads, splits, 2), dtype=torch.float32, device=q.device)
+    blocks = splits + (1 if keep_first else 0)         # the kept first keys are the work of one more block
+    partial_o = torch.empty((T, num_heads, blocks, value_dim), dtype=torch.float32, device=q.device)
+    partial_ml = torch.empty((T, num_heads, blocks, 2), dtype=torch.float32, device=q.device)
     _check(_fn("attention", "mi_decode_attention_forms")(
         _p(q), q_ld, T, num_heads, num_kv_heads, head_dim, value_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
         _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale), int(window or 0),
         split_keys, splits, _p(partial_o), _p(partial_ml), _p(out), out_ld, _p(head_scales), _p(score_bias),
-        1 if sigmoid else 0, _stream()), "decode_attention")
+        1 if sigmoid else 0, int(keep_first), _p(sinks), _stream()), "decode_attention")
 
 
 # --------------------------------------------------------------------------- mamba2

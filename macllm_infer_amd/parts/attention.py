@@ -125,6 +125,10 @@ class Attention(Mixer):
         f32 = lambda name: get(name).to(torch.float32).contiguous().to(build.device)
         self.sink = f32("sink") if spec.sink else None
         self.fixed_sink = spec.fixed_sink
+        # a sink of a fixed score is, to the kernels, a sink tensor with that score for every head
+        self.sinks = self.sink
+        if spec.fixed_sink is not None:
+            self.sinks = torch.full((spec.num_heads,), float(spec.fixed_sink), dtype=torch.float32, device=build.device)
         self.keep_first = int(spec.keep_first) if spec.window else 0
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))
         # the forms that ``ops.attention_prepare`` and the general kernel's extra terms serve
@@ -276,25 +280,26 @@ class Attention(Mixer):
         if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
             tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
         plain = not sigmoid and self.head_scales is None and spec.value_width == spec.head_dim
-        if self.keep_first > 0 or self.fixed_sink is not None:
-            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
-                                step.lane_of_token, step.positions, spec.scale, spec.window, out, step.max_seq_len,
-                                value_dim=spec.value_width, head_scales=self.head_scales, keep_first=self.keep_first,
-                                fixed_sink=self.fixed_sink, **tiles)
-            return
         aligned = (qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 and out.stride(0) % 4 == 0
                    and out.data_ptr() % 8 == 0)
+        kept, sinks = self.keep_first, self.sinks
         if (step.max_query_len == 1 and aligned
-                and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2], spec.value_width)):
+                and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2], spec.value_width, kept)):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                  step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len, out,
                                  value_dim=spec.value_width, head_scales=self.head_scales, score_bias=self.score_bias,
-                                 sigmoid=sigmoid)
+                                 sigmoid=sigmoid, keep_first=kept, sinks=sinks)
         elif (plain and tiles and aligned and step.query_tile == self.query_tile
                 and ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2])):
             ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                   step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window, out,
-                                  step.max_seq_len)
+                                  step.max_seq_len, sinks=sinks, keep_first=kept)
+        elif kept > 0 or sinks is not None:
+            # the general kernel knows every form
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, out, step.max_seq_len,
+                                sinks=sinks, value_dim=spec.value_width, head_scales=self.head_scales,
+                                keep_first=kept, **tiles)
         elif (tiles and aligned and step.query_tile == self.query_tile
                 and ops.prefill_attention_forms_supported(qkv.dtype, *geometry, spec.value_width, cache.k_cache.shape[2],
                                                           sigmoid, self.head_scales is not None)):

@@ -41,8 +41,9 @@ class Mamba2(Mixer):
             out += [Expect(f"{prefix}.in_proj.bias", ((spec.projection_width,),), init="bias"),
                     Expect(f"{prefix}.out_proj.bias", ((hidden_size,),), init="bias")]
         if spec.gated_norm:
-            out.append(Expect(f"{prefix}.norm.weight",
-                              ((spec.inner_size,), (spec.norm_parts, spec.inner_size // spec.norm_parts)),
+            grouped, flat = (spec.norm_parts, spec.inner_size // spec.norm_parts), (spec.inner_size,)
+            # stored by group where the norm's parts are the scan's groups, flat where they are given on their own
+            out.append(Expect(f"{prefix}.norm.weight", (grouped, flat) if spec.norm_groups is None else (flat, grouped),
                               init="norm"))
         return out
 

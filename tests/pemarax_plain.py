@@ -12,6 +12,40 @@ import torch
 
 F64 = torch.float64
 
+# Rounding of activations, for measuring what 16-bit rounding alone does to a model: None (exact), or a function
+# that rounds a float64 tensor the way a 16-bit engine rounds its activations (see ``activations_rounded``).
+_ROUND = None
+
+
+def rnd(x):
+    return x if _ROUND is None else _ROUND(x)
+
+
+class activations_rounded:
+    """Within the block the plain model rounds its activations to bfloat16 where a 16-bit engine holds them in 16
+    bits (projections' outputs, normed rows, convolutions, attended heads, expert rows).  With a generator the
+    rounding is dithered (up or down at random, in proportion), so that several runs are several samples."""
+
+    def __init__(self, generator=None):
+        self.generator = generator
+
+    def _round(self, x):
+        if self.generator is None:
+            return x.to(torch.bfloat16).to(F64)
+        low = (x.to(torch.float32).view(torch.int32) & -65536).view(torch.float32).to(F64)      # toward zero
+        step = (low.abs() * 2.0 ** -7).clamp(min=1e-30)
+        share = ((x - low).abs() / step).clamp(0.0, 1.0)
+        up = torch.rand(x.shape, generator=self.generator, dtype=F64) < share
+        return torch.where(up, (low + torch.sign(x) * step), low).to(torch.bfloat16).to(F64)
+
+    def __enter__(self):
+        global _ROUND
+        self.before, _ROUND = _ROUND, self._round
+
+    def __exit__(self, *exc):
+        global _ROUND
+        _ROUND = self.before
+
 
 def rms_unit(x, eps):
     """x divided by its root mean square over the last dimension, eps inside the root."""
@@ -105,54 +139,54 @@ def attention_mixer(h, m, w, eps):
     norms of q and k, a window that keeps the first tokens, a sink in the softmax."""
     T = h.shape[0]
     H, G, dim, vdim = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q, k, v = h @ w["q"].T, h @ w["k"].T, h @ w["v"].T
+    q, k, v = rnd(h @ w["q"].T), rnd(h @ w["k"].T), rnd(h @ w["v"].T)
     if m.get("conv"):
-        q, k, v = causal_conv(q, w["q.conv"]), causal_conv(k, w["k.conv"]), causal_conv(v, w["v.conv"])
+        q, k, v = rnd(causal_conv(q, w["q.conv"])), rnd(causal_conv(k, w["k.conv"])), rnd(causal_conv(v, w["v.conv"]))
     q, k, v = q.view(T, H, dim), k.view(T, G, dim), v.view(T, G, vdim)
     positions = torch.arange(T)
     if m.get("rot"):
         f, magnitude = rotary_frequencies(m["rot"]["base"], m["rot"]["dims"], m["rot"].get("scaling"))
         q = rotate(q, positions, f, m["rot"]["dims"], True, magnitude)
         k = rotate(k, positions, f, m["rot"]["dims"], True, magnitude)
-    q, k = rms_unit(q, eps), rms_unit(k, eps)
+    q, k = rnd(rms_unit(q, eps)), rnd(rms_unit(k, eps))
     k = k.repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
     scores = torch.einsum("thd,shd->hts", q, k) * m["scale"]
     seen = visible(T, m["mask"]["size"], m["mask"].get("keep_first", 0))
-    return weighted_values(scores, seen, v, sink=True).reshape(T, H * vdim) @ w["o"].T
+    return rnd(rnd(weighted_values(scores, seen, v, sink=True).reshape(T, H * vdim)) @ w["o"].T)
 
 
 def latent_attention_mixer(h, m, w, eps):
     T = h.shape[0]
     H, dim, rot_dim, vdim, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    q = (h @ w["q"].T).view(T, H, dim + rot_dim)
-    down = h @ w["dkv"].T
-    c = rms_unit(down[:, :rank], eps) * w["dkv.norm"]
+    q = rnd(h @ w["q"].T).view(T, H, dim + rot_dim)
+    down = rnd(h @ w["dkv"].T)
+    c = rnd(rms_unit(down[:, :rank], eps) * w["dkv.norm"])
     shared = down[:, rank:].view(T, 1, rot_dim)
     positions = torch.arange(T)
     q_plain, q_turned = q[..., :dim], q[..., dim:]
     if rot_dim:
         f, _ = rotary_frequencies(m["rot"]["base"], m["rot"]["dims"])
-        q_turned = rotate(q_turned, positions, f, m["rot"]["dims"], False)
-        shared = rotate(shared, positions, f, m["rot"]["dims"], False)
+        q_turned = rnd(rotate(q_turned, positions, f, m["rot"]["dims"], False))
+        shared = rnd(rotate(shared, positions, f, m["rot"]["dims"], False))
     keys = (c @ w["uk"].T).view(T, H, dim)
     values = (c @ w["uv"].T).view(T, H, vdim)
     scores = torch.einsum("thd,shd->hts", q_plain, keys) + torch.einsum("thd,sd->hts", q_turned, shared[:, 0])
     seen = visible(T, m["mask"]["size"])
-    return weighted_values(scores * m["scale"], seen, values, sink=False).reshape(T, H * vdim) @ w["o"].T
+    return rnd(rnd(weighted_values(scores * m["scale"], seen, values, sink=False).reshape(T, H * vdim)) @ w["o"].T)
 
 
 def windowed_attention(h, m, w, eps):
     """The left half of ``parallel``: normed queries and keys (one weight for all heads), no rotation."""
     T = h.shape[0]
     H, G, dim, vdim = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = rms_unit((h @ w["q"].T).view(T, H, dim), eps) * w["q.norm"]
-    k = rms_unit((h @ w["k"].T).view(T, G, dim), eps) * w["k.norm"]
-    v = (h @ w["v"].T).view(T, G, vdim)
+    q = rnd(rms_unit(rnd(h @ w["q"].T).view(T, H, dim), eps) * w["q.norm"])
+    k = rnd(rms_unit(rnd(h @ w["k"].T).view(T, G, dim), eps) * w["k.norm"])
+    v = rnd(h @ w["v"].T).view(T, G, vdim)
     k = k.repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
     scores = torch.einsum("thd,shd->hts", q, k) * m["scale"]
-    return weighted_values(scores, visible(T, m["mask"]["size"]), v, sink=False).reshape(T, H * vdim) @ w["o"].T
+    return rnd(rnd(weighted_values(scores, visible(T, m["mask"]["size"]), v, sink=False).reshape(T, H * vdim)) @ w["o"].T)
 
 
 def state_space(h, m, w, eps):
@@ -160,9 +194,9 @@ def state_space(h, m, w, eps):
     T = h.shape[0]
     heads, P, N, groups = m["heads"], m["vdim"], m["state"], m["groups"]
     inner = heads * P
-    u = h @ w["in"].T
+    u = rnd(h @ w["in"].T)
     z, xbc, dt = u[:, :inner], u[:, inner:2 * inner + 2 * groups * N], u[:, 2 * inner + 2 * groups * N:]
-    xbc = silu(causal_conv(xbc, w["conv"], w["conv.b"]))
+    xbc = rnd(silu(causal_conv(xbc, w["conv"], w["conv.b"])))
     x = xbc[:, :inner].view(T, heads, P)
     B = xbc[:, inner:inner + groups * N].view(T, groups, N)
     C = xbc[:, inner + groups * N:].view(T, groups, N)
@@ -179,7 +213,7 @@ def state_space(h, m, w, eps):
     gated = y.reshape(T, inner) * silu(z)
     parts = m.get("norm_groups", 1)
     normed = rms_unit(gated.view(T, parts, inner // parts), eps).reshape(T, inner) * w["norm"]
-    return normed @ w["o"].T
+    return rnd(rnd(normed) @ w["o"].T)
 
 
 def parallel_mixer(h, m, w, eps):
@@ -205,7 +239,7 @@ def mixture(h, mlp, w):
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, weight in zip(experts[t].tolist(), weights[t]):
-            inner = torch.relu(w[f"e{e}.up"] @ h[t]) ** 2
+            inner = rnd(torch.relu(w[f"e{e}.up"] @ h[t]) ** 2)
             out[t] = out[t] + weight * (w[f"e{e}.down"] @ inner)
     return out
 
@@ -225,13 +259,13 @@ def forward(config, tensors, tokens, streams=False):
     for index, layer in enumerate(config["layers"]):
         w = layer_tensors(tensors, f"l{index}.")
         mix = layer_tensors(tensors, f"l{index}.mix.")
-        normed = rms_unit(x, eps) * (1.0 + w["norm1"])
+        normed = rnd(rms_unit(x, eps) * (1.0 + w["norm1"]))
         x = x + mult * MIXERS[layer["type"]](normed, layer["mixer"], mix, eps)
         if layer.get("mlp") is not None:
-            normed = rms_unit(x, eps) * (1.0 + w["norm2"])
+            normed = rnd(rms_unit(x, eps) * (1.0 + w["norm2"]))
             x = x + mult * mixture(normed, layer["mlp"], layer_tensors(tensors, f"l{index}.mlp."))
         behind.append(x.clone())
-    final = rms_unit(x, eps) * (1.0 + tensors["final.norm"].to(F64))
+    final = rnd(rms_unit(x, eps) * (1.0 + tensors["final.norm"].to(F64)))
     logits = final @ tensors["head"].to(F64).T
     return (logits, behind) if streams else logits
 
@@ -244,11 +278,24 @@ def choice_margins(config, tensors, tokens):
     least = torch.full((x.shape[0],), float("inf"), dtype=F64)
     for index, layer in enumerate(config["layers"]):
         w = layer_tensors(tensors, f"l{index}.")
-        normed = rms_unit(x, eps) * (1.0 + w["norm1"])
+        normed = rnd(rms_unit(x, eps) * (1.0 + w["norm1"]))
         x = x + mult * MIXERS[layer["type"]](normed, layer["mixer"], layer_tensors(tensors, f"l{index}.mix."), eps)
         if layer.get("mlp") is not None:
-            normed = rms_unit(x, eps) * (1.0 + w["norm2"])
+            normed = rnd(rms_unit(x, eps) * (1.0 + w["norm2"]))
             mlp = layer_tensors(tensors, f"l{index}.mlp.")
             least = torch.minimum(least, router_choice(normed, layer["mlp"], mlp)[2])
             x = x + mult * mixture(normed, layer["mlp"], mlp)
     return least
+
+
+def rounding_noise(config, tensors, tokens, samples=4, seed=1):
+    """Per position, how far 16-bit rounding of the activations alone moves the plain model's logits (max-abs over
+    the vocabulary, the largest of ``samples`` dithered runs and one that rounds to nearest)."""
+    exact = forward(config, tensors, tokens)
+    generator = torch.Generator().manual_seed(seed)
+    worst = torch.zeros(exact.shape[0], dtype=F64)
+    for sample in range(samples + 1):
+        with activations_rounded(generator if sample else None):
+            moved = forward(config, tensors, tokens)
+        worst = torch.maximum(worst, (moved - exact).abs().max(dim=-1).values)
+    return worst

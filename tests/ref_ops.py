@@ -218,7 +218,7 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
             out[token, head * value_dim:(head + 1) * value_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
 
 
-def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim=None):
+def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size, value_dim=None, keep_first=0):
     return False
 
 
@@ -227,10 +227,11 @@ def prefill_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_s
 
 
 def decode_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
-                     scale, window, max_seq_len, out, value_dim=None, head_scales=None, score_bias=None, sigmoid=False):
+                     scale, window, max_seq_len, out, value_dim=None, head_scales=None, score_bias=None, sigmoid=False,
+                     keep_first=0, sinks=None):
     paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
                     scale, window, out, value_dim=value_dim, head_scales=head_scales, score_bias=score_bias,
-                    sigmoid=sigmoid)
+                    sigmoid=sigmoid, keep_first=keep_first, sinks=sinks)
 
 
 def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out, activation=True):
