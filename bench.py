@@ -4,7 +4,7 @@ MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
     python bench.py --workload serving [--shape 0.5b|7b|34b]
     python bench.py --microbench
-    python bench.py --design mukutar|lutosun|motolix [--shape 0.5b|7b] [--layers L] [--window W] [--only DESIGN|falcon_h1]
+    python bench.py --design mukutar|lutosun|motolix|pemarax [--shape 0.5b|7b] [--layers L] [--window W] [--only DESIGN|falcon_h1]
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
@@ -34,7 +34,11 @@ feed-forward width: for both the 2,048-token prompt step and decode steps at bat
 a shared one, layer norms, a hashed bigram embedding), and ``--design motolix`` for a Motolix-shaped one (two layers
 in three softmax attention with normed projections and turned values beside gated linear attention, the third sigmoid
 attention whose values are its keys; a norm before and behind every branch; GELU-gated feed-forwards; the middle
-third of the layers run twice).  The default workload and its line are not touched by any of them.
+third of the layers run twice), and ``--design pemarax`` for a Pemarax-shaped one (layers in turn: attention with
+convolutions behind its projections, kept first tokens and a sink; two of windowed latent attention; windowed
+attention beside a Mamba-2 mixer, their outputs normed each; experts without a gate on every layer), with
+``--beside lutosun`` beside the Lutosun-shaped model of equal sizes instead of the Falcon-H1 shape.  The default
+workload and its line are not touched by any of them.
 
 ``--workload serving`` runs whole requests through the scheduler and the sampler instead
 (``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
@@ -198,11 +202,40 @@ def motolix_shape(shape: dict, layers: int) -> dict:
             "layers": [dict(kinds[index % 3], mlp=mlp) for index in range(stored)]}
 
 
+def pemarax_shape(shape: dict, layers: int, window: int) -> dict:
+    """A Pemarax configuration with the sizes of a Falcon-H1 ``shape``: the same width, vocabulary, heads and head
+    size.  Layers in turn: attention (convolutions of three taps behind its projections, ramp-scaled rotation, the
+    first four tokens kept behind the window), two of latent attention (a latent of two heads' width as far as a
+    cached row's 256 numbers allow, half a head turned), and a parallel layer (attention with values twice as wide
+    as its keys beside a state-space mixer of the shape's own sizes); every layer with sixteen experts half as wide
+    as the shape's feed-forward, of which a token uses three (the experts have no gate: as many products a token as
+    the dense feed-forward)."""
+    width, dim = shape["hidden_size"], shape["head_dim"]
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    attention = {"type": "attention", "mixer": {
+        "conv": 3, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 8.0 / dim,
+        "mask": {"size": window, "keep_first": 4},
+        "rot": {"base": 5e5, "dims": dim, "scaling": {"factor": 4.0, "original": 512, "fast": 32.0, "slow": 1.0}}}}
+    turned = dim // 2
+    latent = {"type": "latent_attention", "mixer": {
+        "heads": heads, "dim": dim, "rot_dim": turned, "vdim": dim + dim // 4, "kv_rank": min(2 * dim, 256 - turned),
+        "rot": {"base": 5e5, "dims": turned}, "scale": (dim + turned) ** -0.5, "mask": {"size": window}}}
+    parallel = {"type": "parallel", "mixer": {
+        "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": 2 * dim, "scale": dim ** -0.5,
+                 "mask": {"size": max(window // 2, 1)}},
+        "right": {"conv": shape["mamba_d_conv"], "groups": shape["mamba_n_groups"], "heads": shape["mamba_n_heads"],
+                  "norm_groups": 1, "state": shape["mamba_d_state"], "vdim": shape["mamba_d_head"]}}}
+    kinds = (attention, latent, latent, parallel)
+    mlp = {"kind": "moe", "expert": {"ff": shape["intermediate_size"] // 2}, "router": {"experts": 16, "top": 3}}
+    return {"architecture": "Pemarax", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
+            "residual_mult": 0.5, "layers": [dict(kinds[index % 4], mlp=mlp) for index in range(layers)]}
+
+
 def design_points(args) -> int:
     """Prompt and decode steps of a model of another design with the sizes of a Falcon-H1 shape, and of that shape."""
     import torch
     from macllm_infer_amd import Engine, Lane
-    from macllm_infer_amd.config import FalconH1Config, LutosunConfig, MotolixConfig, MukutarConfig
+    from macllm_infer_amd.config import FalconH1Config, LutosunConfig, MotolixConfig, MukutarConfig, PemaraxConfig
     from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
     from macllm_infer_amd.weights.random_init import random_tensors
 
@@ -214,9 +247,14 @@ def design_points(args) -> int:
         configs = {"lutosun": LutosunConfig.from_dict(lutosun_shape(shape, layers))}
     elif args.design == "motolix":
         configs = {"motolix": MotolixConfig.from_dict(motolix_shape(shape, layers))}
+    elif args.design == "pemarax":
+        configs = {"pemarax": PemaraxConfig.from_dict(pemarax_shape(shape, layers, args.window))}
+        if args.beside == "lutosun":         # the closest of the other designs: latent attention and routed experts
+            configs["lutosun"] = LutosunConfig.from_dict(lutosun_shape(shape, layers))
     else:
         configs = {"mukutar": MukutarConfig.from_dict(mukutar_shape(shape, layers, args.window))}
-    configs["falcon_h1"] = FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))
+    if "lutosun" not in configs or args.design == "lutosun":
+        configs["falcon_h1"] = FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))
     batches = [] if args.prefill_only else ([args.batch] if args.skip_points else sorted({1, args.batch, 64}))
     largest = max(batches, default=1)
     per_request = -(-(CONTEXT + args.steps + args.warmup + 1) // 64) * 64
@@ -368,11 +406,15 @@ def main() -> int:
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     parser.add_argument("--microbench", action="store_true",
                         help="only this GPU's streaming read and read-modify-write bandwidth")
-    parser.add_argument("--design", default=None, choices=["mukutar", "lutosun", "motolix"],
+    parser.add_argument("--design", default=None, choices=["mukutar", "lutosun", "motolix", "pemarax"],
                         help="measure a model of this design with the sizes of --shape (12 layers unless --layers) beside "
                              "the Falcon-H1 shape of equal sizes, instead of the headline workload")
     parser.add_argument("--window", type=int, default=1024, help="--design: the attention layers' window")
-    parser.add_argument("--only", default=None, choices=["mukutar", "lutosun", "motolix", "falcon_h1"], help="--design: one of the two models")
+    parser.add_argument("--only", default=None, choices=["mukutar", "lutosun", "motolix", "pemarax", "falcon_h1"],
+                        help="--design: one of the two models")
+    parser.add_argument("--beside", default="falcon_h1", choices=["falcon_h1", "lutosun"],
+                        help="--design pemarax: the model measured beside it (the Falcon-H1 shape, or the Lutosun-shaped "
+                             "model of equal sizes, the closest of the other designs)")
     parser.add_argument("--write-config", default=None, metavar="PATH",
                         help="write the config.json of --shape / --layers there and exit (what "
                              "utils.kernel_trace --config reads)")
@@ -391,6 +433,8 @@ def main() -> int:
                 json.dump(lutosun_shape(shape, args.layers or 12), handle)
             elif args.design == "motolix" and args.only != "falcon_h1":
                 json.dump(motolix_shape(shape, args.layers or 12), handle)
+            elif args.design == "pemarax" and args.only != "falcon_h1":
+                json.dump(pemarax_shape(shape, args.layers or 12, args.window), handle)
             else:
                 layers = args.layers or (12 if args.design else shape["num_hidden_layers"])
                 json.dump(dict(shape, num_hidden_layers=layers), handle)

@@ -62,7 +62,7 @@ extern "C" int mi_feed_tokens(int* token_ids, int tokens, const int* source, int
 }
 
 // ---------------------------------------------------------------- add + rmsnorm
-// For each processed row r:  v = h[r] (+ delta0[r]) (+ delta1[r]);  if update: h[r] = v;
+// For each processed row r:  v = h[r] (+ factor0 * delta0[r]) (+ factor1 * delta1[r]);  if update: h[r] = v;
 // out[i] = v / sqrt(mean(v^2) + eps) * weight.
 // With `rows` the kernel processes h[rows[i]] and writes out[i] (h is not updated).
 // The sum of squares is accumulated in float32 in an order fixed by (d, blockDim) alone,
@@ -70,7 +70,8 @@ extern "C" int mi_feed_tokens(int* token_ids, int tokens, const int* source, int
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta0,
                                    const TD* __restrict__ delta1, const float* __restrict__ weight, float eps,
-                                   TO* __restrict__ out, const int* __restrict__ rows, int d) {
+                                   TO* __restrict__ out, const int* __restrict__ rows, int d, float factor0,
+                                   float factor1) {
   extern __shared__ float row_values[];
   __shared__ float scratch[16];
   const long out_row = blockIdx.x;
@@ -79,8 +80,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   float sum_squares = 0.f;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = hr[i];
-    if (delta0) v += to_float(delta0[row * d + i]);
-    if (delta1) v += to_float(delta1[row * d + i]);
+    if (delta0) v = fmaf(factor0, to_float(delta0[row * d + i]), v);
+    if (delta1) v = fmaf(factor1, to_float(delta1[row * d + i]), v);
     if (!rows && (delta0 || delta1)) hr[i] = v;
     row_values[i] = v;
     sum_squares += v * v;
@@ -106,7 +107,7 @@ template <typename TD, typename TO, int ROUNDS>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, const TD* __restrict__ delta1,
                        const float* __restrict__ weight, float eps, TO* __restrict__ out,
-                       const int* __restrict__ rows, int d) {
+                       const int* __restrict__ rows, int d, float factor0, float factor1) {
   typedef typename Vec4<float>::type f4;
   typedef typename Vec4<TD>::type d4;
   typedef typename Vec4<TO>::type o4;
@@ -138,8 +139,8 @@ add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, con
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float value = v[r][j];
-      if (delta0) value += (float)a[r][j];
-      if (delta1) value += (float)b[r][j];
+      if (delta0) value = fmaf(factor0, (float)a[r][j], value);        // a factor of one adds the delta as it is
+      if (delta1) value = fmaf(factor1, (float)b[r][j], value);
       v[r][j] = value;
       if (mine) sum_squares += value * value;
     }
@@ -231,7 +232,7 @@ extern "C" int mi_add_partials_rmsnorm(float* h, const float* partial, int S, co
 
 extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, int delta_dtype,
                               const float* weight, float eps, void* out, int out_dtype, const int* rows,
-                              int n_rows, int d, hipStream_t stream) {
+                              int n_rows, int d, float factor0, float factor1, hipStream_t stream) {
   if (n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
   const bool vectors = d % 4 == 0 && d <= 256 * 4 * NORM_MAX_ROUNDS && ((uintptr_t)h % 16) == 0 &&
                        ((uintptr_t)delta0 % 16) == 0 && ((uintptr_t)delta1 % 16) == 0 &&
@@ -242,19 +243,19 @@ extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, 
   do {                                                                                                      \
     if (vectors && d <= 1024)                                                                               \
       add_rmsnorm_vec_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
-                                                                    weight, eps, (TO*)out, rows, d);        \
+                                                                    weight, eps, (TO*)out, rows, d, factor0, factor1); \
     else if (vectors && d <= 2048)                                                                          \
       add_rmsnorm_vec_kernel<TD, TO, 2><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
-                                                                    weight, eps, (TO*)out, rows, d);        \
+                                                                    weight, eps, (TO*)out, rows, d, factor0, factor1); \
     else if (vectors && d <= 4096)                                                                          \
       add_rmsnorm_vec_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
-                                                                    weight, eps, (TO*)out, rows, d);        \
+                                                                    weight, eps, (TO*)out, rows, d, factor0, factor1); \
     else if (vectors)                                                                                       \
       add_rmsnorm_vec_kernel<TD, TO, NORM_MAX_ROUNDS><<<n_rows, 256, 0, stream>>>(                          \
-          h, (const TD*)delta0, (const TD*)delta1, weight, eps, (TO*)out, rows, d);                         \
+          h, (const TD*)delta0, (const TD*)delta1, weight, eps, (TO*)out, rows, d, factor0, factor1);       \
     else                                                                                                    \
       add_rmsnorm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta0, (const TD*)delta1,     \
-                                                               weight, eps, (TO*)out, rows, d);             \
+                                                               weight, eps, (TO*)out, rows, d, factor0, factor1); \
   } while (0)
   if (delta_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
   else if (delta_dtype == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
@@ -311,6 +312,58 @@ normed_sum_kernel(NormedSumBranches branches, int count, float* __restrict__ out
   }
 }
 
+// The same for rows of up to 256 * ROUNDS numbers: a thread asks for all its elements of every branch at once and
+// keeps them in registers, the branches' sums of squares cross the workgroup together (one barrier), and the row
+// is read once.  A step of a few rows is a chain of waits, and this takes most of them out.
+template <int ROUNDS>
+__global__ void __launch_bounds__(256)
+normed_sum_rows_kernel(NormedSumBranches branches, int count, float* __restrict__ out, int d) {
+  __shared__ float sums[256 / WAVE][NORMED_SUM_MOST];
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  float values[NORMED_SUM_MOST][ROUNDS];
+#pragma unroll
+  for (int b = 0; b < NORMED_SUM_MOST; ++b) {
+    const int from = b < count ? b : 0;           // an absent branch reads the first again and is dropped
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int i = min((int)threadIdx.x + 256 * r, d - 1);
+      values[b][r] = branches.is_bf16[from] ? to_float(((const bf16_t*)branches.rows[from])[row * branches.ld[from] + i])
+                                            : ((const float*)branches.rows[from])[row * branches.ld[from] + i];
+    }
+  }
+  float squares[NORMED_SUM_MOST];
+#pragma unroll
+  for (int b = 0; b < NORMED_SUM_MOST; ++b) {
+    squares[b] = 0.f;
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r)
+      if ((int)threadIdx.x + 256 * r < d) squares[b] = fmaf(values[b][r], values[b][r], squares[b]);
+    squares[b] = wave_sum(squares[b]);
+    if (lane == 0) sums[wave][b] = squares[b];
+  }
+  __syncthreads();
+  float scale[NORMED_SUM_MOST];
+#pragma unroll
+  for (int b = 0; b < NORMED_SUM_MOST; ++b) {
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 256 / WAVE; ++w) total += sums[w][b];
+    scale[b] = b < count ? branches.factor[b] / sqrtf(total / (float)d + branches.eps[b]) : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int i = (int)threadIdx.x + 256 * r;
+    if (i >= d) break;
+    float sum = 0.f;
+#pragma unroll
+    for (int b = 0; b < NORMED_SUM_MOST; ++b)
+      if (b < count) sum = fmaf(values[b][r] * scale[b], branches.weight[b][i], sum);
+    out[row * d + i] = sum;
+  }
+}
+
 extern "C" int mi_normed_sum(const void* const* rows, const int* dtypes, const long* lds, const float* const* weights,
                              const float* factors, const float* eps, int count, float* out, int T, int d,
                              hipStream_t stream) {
@@ -329,7 +382,9 @@ extern "C" int mi_normed_sum(const void* const* rows, const int* dtypes, const l
     branches.is_bf16[b] = dtypes[from] == DT_BF16;
     branches.ld[b] = lds[from];
   }
-  normed_sum_kernel<<<T, 256, 0, stream>>>(branches, count, out, d);
+  if (d <= 256 * 4) normed_sum_rows_kernel<4><<<T, 256, 0, stream>>>(branches, count, out, d);
+  else if (d <= 256 * 16) normed_sum_rows_kernel<16><<<T, 256, 0, stream>>>(branches, count, out, d);
+  else normed_sum_kernel<<<T, 256, 0, stream>>>(branches, count, out, d);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

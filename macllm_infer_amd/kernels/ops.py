@@ -33,7 +33,7 @@ _SIGNATURES = {
         "mi_embed": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_feed_tokens": [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
         "mi_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
-                           _c_int, _c_ptr],
+                           _c_int, _c_float, _c_float, _c_ptr],
         "mi_add_partials_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
                                     _c_int, _c_ptr],
         "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -274,8 +274,10 @@ def feed_tokens(token_ids: torch.Tensor, source: torch.Tensor, dst: Sequence[int
 
 
 def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.Tensor, eps: float,
-                out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
-    """h += sum(deltas) (float32, in place); out = h / sqrt(mean(h^2) + eps) * weight.
+                out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                factors: Optional[Sequence[float]] = None) -> None:
+    """h += sum(deltas) (float32, in place); out = h / sqrt(mean(h^2) + eps) * weight.  With ``factors`` (a number
+    for each delta) h += sum of factor * delta, the products in float32.
 
     With ``rows`` (int32 indices) only those rows are read, ``out[i]`` gets row ``rows[i]``
     and ``h`` is left as it is.  ``out`` may be None when only the sum is wanted."""
@@ -296,9 +298,11 @@ def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.T
         _need(out.shape == (n_rows, d) and out.is_contiguous(), "add_rmsnorm: out must be contiguous [rows, d]")
     delta_dtype = _dt(deltas[0]) if deltas else DT_F32
     out_dtype = _dt(out) if out is not None else DT_F32
+    _need(factors is None or len(factors) == len(deltas), "add_rmsnorm: one factor for each delta")
+    scales = [float(factor) for factor in (factors or ())] + [1.0, 1.0]
     _check(_fn("common", "mi_add_rmsnorm")(
         _p(h), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
-        delta_dtype, _p(weight), float(eps), _p(out), out_dtype, _p(rows), n_rows, d, _stream()),
+        delta_dtype, _p(weight), float(eps), _p(out), out_dtype, _p(rows), n_rows, d, scales[0], scales[1], _stream()),
         "add_rmsnorm", f"(d={d})")
 
 

@@ -43,13 +43,16 @@ def add_normed_branches(h: torch.Tensor, normed: NormedBranches, vector: Optiona
     ops.add_layernorm(h, branches, vector, None, None, 0.0, None, branch_norm=(normed.weight, normed.bias, normed.eps))
 
 
-def fold_weighted(residual: Residual) -> None:
+def fold_weighted(residual: Residual, keep_weighted: bool = False) -> None:
     """Add the ``WeightedBranch``es, ``NormedBranches`` and ``RowVector``s among the pending branches to the stream
-    with the kernel that knows them, and leave the others pending: for a norm whose own kernel fuses none of them."""
+    with the kernel that knows them, and leave the others pending: for a norm whose own kernel fuses none of them
+    (``keep_weighted``: the weighted branches stay pending too, for a norm that adds them itself)."""
     kept = []
     for branch in residual.pending:
         if isinstance(branch, NormedBranches):
             add_normed_branches(residual.h, branch)
+        elif isinstance(branch, WeightedBranch) and keep_weighted:
+            kept.append(branch)
         elif isinstance(branch, WeightedBranch):
             ops.stream_add(residual.h, branch.rows, branch.factor, None)
         elif isinstance(branch, RowVector):
@@ -103,8 +106,13 @@ class RmsNorm(Part):
     def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add the pending branch outputs to the residual stream and return its normed rows
         (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""
-        if any(isinstance(branch, (WeightedBranch, RowVector, NormedBranches)) for branch in residual.pending):
-            fold_weighted(residual)
+        if any(isinstance(branch, (RowVector, NormedBranches)) for branch in residual.pending):
+            fold_weighted(residual, keep_weighted=True)
+        if any(isinstance(branch, WeightedBranch) for branch in residual.pending):
+            if any(isinstance(branch, ScaledBranch) for branch in residual.pending):
+                fold_weighted(residual)
+            else:
+                return self._forward_weighted(residual, rows)
         pending = residual.pending
         slab = partial_slab(pending)
         if slab is not None and slab.shape[0] <= 16 and residual.h.shape[1] % 4 == 0:
@@ -139,6 +147,24 @@ class RmsNorm(Part):
         ops.add_rmsnorm(residual.h, pending, self.weight, self.eps, out, rows)
         if rows is None:
             residual.pending = []
+        return out
+
+
+    def _forward_weighted(self, residual: Residual, rows: Optional[torch.Tensor]) -> torch.Tensor:
+        """Branches that join the stream times a number each: the norm's kernel adds up to two of one dtype with
+        their factors in its own launch (the products in float32); what is left over is added before."""
+        pairs = [(branch.rows, float(branch.factor)) if isinstance(branch, WeightedBranch) else (branch, 1.0)
+                 for branch in residual.pending]
+        pairs = [(tensor if tensor.is_contiguous() else tensor.contiguous(), factor) for tensor, factor in pairs]
+        while len(pairs) > 2 or (len(pairs) == 2 and pairs[0][0].dtype != pairs[1][0].dtype):
+            tensor, factor = pairs.pop(0)
+            ops.stream_add(residual.h, tensor, factor, None)
+        count = residual.h.shape[0] if rows is None else rows.numel()
+        out = torch.empty((count, residual.h.shape[1]), dtype=self.build.dtype, device=residual.h.device)
+        ops.add_rmsnorm(residual.h, [tensor for tensor, _ in pairs], self.weight, self.eps, out, rows,
+                        factors=[factor for _, factor in pairs])
+        # with a gather the stream itself was not changed by the norm's kernel: its branches stay pending
+        residual.pending = [] if rows is None else [WeightedBranch(tensor, factor) for tensor, factor in pairs]
         return out
 
 

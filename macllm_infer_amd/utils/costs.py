@@ -57,6 +57,8 @@ def model_sizes(spec) -> dict:
                                          (kv + values) if entry.kv_from is None else 0, part.window))
                 total["mixed"] += mixed
                 total["in_width"] += q + kv + projected
+                if getattr(part, "conv_kernel", 0) > 1:                    # the tail of the projections' convolution
+                    total["conv_tail"] += (part.conv_kernel - 1) * (q + kv + projected)
             elif part.kind == "gated_linear_attention":
                 keys, values = part.num_heads * part.key_dim, part.num_heads * part.value_dim
                 rank = part.decay_rank or 16
@@ -70,7 +72,10 @@ def model_sizes(spec) -> dict:
                 heads, rank, turned = part.num_heads, part.kv_rank, part.rope_dim
                 q = heads * (part.head_dim + turned)
                 # down-projections, the queries' up-projection and their way into the latent space; out of it and out
-                total["in_weights"] += (part.q_rank + rank + turned) * d + q * part.q_rank + heads * part.head_dim * rank
+                if part.q_rank is None:                                    # the queries projected directly
+                    total["in_weights"] += (q + rank + turned) * d + heads * part.head_dim * rank
+                else:
+                    total["in_weights"] += (part.q_rank + rank + turned) * d + q * part.q_rank + heads * part.head_dim * rank
                 total["out_weights"] += heads * part.value_dim * rank + d * heads * part.value_dim
                 cached = (rank + turned) if entry.kv_from is None else 0        # one latent and one turned part a token
                 total["kv_per_token"] += cached
@@ -78,7 +83,7 @@ def model_sizes(spec) -> dict:
                 total["attention"] += heads * (2 * rank + turned) / 2.0
                 total["windows"].append((heads * (2 * rank + turned) / 2.0, cached, part.window))
                 total["mixed"] += heads * part.value_dim + heads * rank
-                total["in_width"] += part.q_rank + rank + turned + q + heads * (rank + turned)
+                total["in_width"] += (part.q_rank or 0) + rank + turned + q + heads * (rank + turned)
             elif part.kind == "retention":
                 keys, values = part.num_heads * part.key_dim, part.num_heads * part.value_dim
                 total["in_weights"] += (2 * keys + 2 * values) * d
@@ -118,7 +123,8 @@ def model_sizes(spec) -> dict:
             total["gate_up"] += (ffn.num_experts + (1 if shared else 0)) * d + 2 * shared * d
             total["down"] += d * shared
             total["inner"] += shared + ffn.top_k * ffn.expert_size
-            total["experts"].append((ffn.num_experts, ffn.top_k, 2 * ffn.expert_size * d, d * ffn.expert_size))
+            first = (2 if getattr(ffn.activation, "gated", True) else 1) * ffn.expert_size * d      # gate and up, or up alone
+            total["experts"].append((ffn.num_experts, ffn.top_k, first, d * ffn.expert_size))
         elif layer.ffn.kind == "polynorm_ffn":
             total["gate_up"] += layer.ffn.intermediate_size * d
             total["down"] += d * layer.ffn.intermediate_size

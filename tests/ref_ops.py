@@ -25,10 +25,10 @@ def feed_tokens(token_ids, source, dst, src):
         token_ids[int(place)] = source[int(row)]
 
 
-def add_rmsnorm(h, deltas, weight, eps, out, rows=None):
+def add_rmsnorm(h, deltas, weight, eps, out, rows=None, factors=None):
     total = h.clone()
-    for delta in deltas:
-        total += _f(delta)
+    for index, delta in enumerate(deltas):
+        total += _f(delta) * (1.0 if factors is None else float(factors[index]))
     if rows is None:
         if deltas:
             h.copy_(total)
