@@ -312,13 +312,13 @@ normed_sum_kernel(NormedSumBranches branches, int count, float* __restrict__ out
   }
 }
 
-// The same for rows of up to 256 * ROUNDS numbers: a thread asks for all its elements of every branch at once and
+// The same for rows of up to THREADS * ROUNDS numbers: a thread asks for all its elements of every branch at once and
 // keeps them in registers, the branches' sums of squares cross the workgroup together (one barrier), and the row
 // is read once.  A step of a few rows is a chain of waits, and this takes most of them out.
-template <int ROUNDS>
-__global__ void __launch_bounds__(256)
+template <int ROUNDS, int THREADS>
+__global__ void __launch_bounds__(THREADS)
 normed_sum_rows_kernel(NormedSumBranches branches, int count, float* __restrict__ out, int d) {
-  __shared__ float sums[256 / WAVE][NORMED_SUM_MOST];
+  __shared__ float sums[THREADS / WAVE][NORMED_SUM_MOST];
   const long row = blockIdx.x;
   const int lane = threadIdx.x & (WAVE - 1);
   const int wave = threadIdx.x / WAVE;
@@ -328,7 +328,7 @@ normed_sum_rows_kernel(NormedSumBranches branches, int count, float* __restrict_
     const int from = b < count ? b : 0;           // an absent branch reads the first again and is dropped
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
-      const int i = min((int)threadIdx.x + 256 * r, d - 1);
+      const int i = min((int)threadIdx.x + THREADS * r, d - 1);
       values[b][r] = branches.is_bf16[from] ? to_float(((const bf16_t*)branches.rows[from])[row * branches.ld[from] + i])
                                             : ((const float*)branches.rows[from])[row * branches.ld[from] + i];
     }
@@ -339,7 +339,7 @@ normed_sum_rows_kernel(NormedSumBranches branches, int count, float* __restrict_
     squares[b] = 0.f;
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r)
-      if ((int)threadIdx.x + 256 * r < d) squares[b] = fmaf(values[b][r], values[b][r], squares[b]);
+      if ((int)threadIdx.x + THREADS * r < d) squares[b] = fmaf(values[b][r], values[b][r], squares[b]);
     squares[b] = wave_sum(squares[b]);
     if (lane == 0) sums[wave][b] = squares[b];
   }
@@ -349,12 +349,12 @@ normed_sum_rows_kernel(NormedSumBranches branches, int count, float* __restrict_
   for (int b = 0; b < NORMED_SUM_MOST; ++b) {
     float total = 0.f;
 #pragma unroll
-    for (int w = 0; w < 256 / WAVE; ++w) total += sums[w][b];
+    for (int w = 0; w < THREADS / WAVE; ++w) total += sums[w][b];
     scale[b] = b < count ? branches.factor[b] / sqrtf(total / (float)d + branches.eps[b]) : 0.f;
   }
 #pragma unroll
   for (int r = 0; r < ROUNDS; ++r) {
-    const int i = (int)threadIdx.x + 256 * r;
+    const int i = (int)threadIdx.x + THREADS * r;
     if (i >= d) break;
     float sum = 0.f;
 #pragma unroll
@@ -382,8 +382,9 @@ extern "C" int mi_normed_sum(const void* const* rows, const int* dtypes, const l
     branches.is_bf16[b] = dtypes[from] == DT_BF16;
     branches.ld[b] = lds[from];
   }
-  if (d <= 256 * 4) normed_sum_rows_kernel<4><<<T, 256, 0, stream>>>(branches, count, out, d);
-  else if (d <= 256 * 16) normed_sum_rows_kernel<16><<<T, 256, 0, stream>>>(branches, count, out, d);
+  if (d <= 256 * 4) normed_sum_rows_kernel<4, 256><<<T, 256, 0, stream>>>(branches, count, out, d);
+  else if (d <= 1024 * 4) normed_sum_rows_kernel<4, 1024><<<T, 1024, 0, stream>>>(branches, count, out, d);
+  else if (d <= 1024 * 8) normed_sum_rows_kernel<8, 1024><<<T, 1024, 0, stream>>>(branches, count, out, d);
   else normed_sum_kernel<<<T, 256, 0, stream>>>(branches, count, out, d);
   RETURN_IF_LAUNCH_FAILED();
   return 0;

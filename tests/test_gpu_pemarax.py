@@ -651,7 +651,7 @@ def same(got, plain, rows, dtype, what):
     rounding (a choice of experts that turns, a gated norm that divides by little), so the gate at a position is what
     rounding alone does to the plain model there: four times that, or 8 % of the scale where that is more; and the
     median position within 3 % of the scale or twice the plain model's median.  A position one of whose choices of
-    experts is decided by less than 0.03 is left out, with the three positions behind it that the convolutions'
+    experts is decided by less than 0.01 is left out, with the three positions behind it that the convolutions'
     taps carry it to (a few samples of the rounding need not turn that choice, the engine's may); at most half of
     the positions are."""
     want = plain.logits[rows]
@@ -663,9 +663,9 @@ def same(got, plain, rows, dtype, what):
         return
     noise = plain.noise[rows]
     error = (got - want).abs().max(dim=-1).values
-    near = plain.margin < 0.03
+    near = plain.margin < 0.01
     for reach in (1, 2, 3):
-        near[reach:] |= plain.margin[:-reach] < 0.03
+        near[reach:] |= plain.margin[:-reach] < 0.01
     close_call = near[rows]
     assert int(close_call.sum()) * 2 <= max(len(rows), 2), f"{what}: too many positions with close choices"
     error = torch.where(close_call, torch.zeros_like(error), error)
