@@ -204,8 +204,8 @@ def motolix_shape(shape: dict, layers: int) -> dict:
 
 def pemarax_shape(shape: dict, layers: int, window: int) -> dict:
     """A Pemarax configuration with the sizes of a Falcon-H1 ``shape``: the same width, vocabulary, heads and head
-    size.  Layers in turn: attention (convolutions of three taps behind its projections, ramp-scaled rotation, the
-    first four tokens kept behind the window), two of latent attention (a latent of two heads' width as far as a
+    size.  Layers in turn: attention (convolutions of four taps behind its projections, ramp-scaled rotation, the
+    first eight tokens kept behind the window), two of latent attention (a latent of two heads' width as far as a
     cached row's 256 numbers allow, half a head turned), and a parallel layer (attention with values twice as wide
     as its keys beside a state-space mixer of the shape's own sizes); every layer with sixteen experts half as wide
     as the shape's feed-forward, of which a token uses three (the experts have no gate: as many products a token as
@@ -213,13 +213,13 @@ def pemarax_shape(shape: dict, layers: int, window: int) -> dict:
     width, dim = shape["hidden_size"], shape["head_dim"]
     heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
     attention = {"type": "attention", "mixer": {
-        "conv": 3, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 8.0 / dim,
-        "mask": {"size": window, "keep_first": 4},
-        "rot": {"base": 5e5, "dims": dim, "scaling": {"factor": 4.0, "original": 512, "fast": 32.0, "slow": 1.0}}}}
+        "conv": 4, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 8.0 / dim,
+        "mask": {"size": window, "keep_first": 8},
+        "rot": {"base": 1e6, "dims": dim, "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}}
     turned = dim // 2
     latent = {"type": "latent_attention", "mixer": {
         "heads": heads, "dim": dim, "rot_dim": turned, "vdim": dim + dim // 4, "kv_rank": min(2 * dim, 256 - turned),
-        "rot": {"base": 5e5, "dims": turned}, "scale": (dim + turned) ** -0.5, "mask": {"size": window}}}
+        "rot": {"base": 1e6, "dims": turned}, "scale": (dim + turned) ** -0.5, "mask": {"size": window}}}
     parallel = {"type": "parallel", "mixer": {
         "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": 2 * dim, "scale": dim ** -0.5,
                  "mask": {"size": max(window // 2, 1)}},
@@ -228,7 +228,7 @@ def pemarax_shape(shape: dict, layers: int, window: int) -> dict:
     kinds = (attention, latent, latent, parallel)
     mlp = {"kind": "moe", "expert": {"ff": shape["intermediate_size"] // 2}, "router": {"experts": 16, "top": 3}}
     return {"architecture": "Pemarax", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
-            "residual_mult": 0.5, "layers": [dict(kinds[index % 4], mlp=mlp) for index in range(layers)]}
+            "residual_mult": 0.7, "layers": [dict(kinds[index % 4], mlp=mlp) for index in range(layers)]}
 
 
 def design_points(args) -> int:

@@ -82,7 +82,7 @@ PEM_B = {
 
 # the head and state sizes that the matrix-core kernels take, so that bfloat16 steps run through them
 PEM_C = {
-    "architecture": "Pemarax", "width": 128, "vocab": 211, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+    "architecture": "Pemarax", "width": 128, "vocab": 211, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
     "layers": [
         with_mlp(attention(4, 2, 64, 64, window=80, keep_first=5, conv=3, rot_dims=64, scaling=(4.0, 128, 16.0, 1.0)), moe(8, 2, 64)),
         with_mlp(latent(4, 32, 32, 48, 64, window=70), moe(8, 2, 64)),

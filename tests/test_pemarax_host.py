@@ -93,7 +93,7 @@ def test_a_broken_configuration_names_its_key(broken, text):
 
 def test_ramp_scaled_frequencies_against_the_plain_ones():
     from macllm_infer_amd.config import RampScalingSpec
-    for base, dims, numbers in ((10000.0, 16, (4.0, 64, 8.0, 1.0)), (777.0, 12, (8.0, 32, 4.0, 0.5)), (500000.0, 64, (4.0, 512, 32.0, 1.0)),
+    for base, dims, numbers in ((10000.0, 16, (4.0, 64, 8.0, 1.0)), (777.0, 12, (8.0, 32, 4.0, 0.5)), (250000.0, 48, (6.0, 1024, 24.0, 2.0)),
                                 (100.0, 8, (2.0, 16, 1.0, 1.0))):
         scaling = RampScalingSpec(*numbers)
         want, magnitude = pemarax_plain.rotary_frequencies(base, dims, dict(zip(("factor", "original", "fast", "slow"), numbers)))
