@@ -823,3 +823,93 @@ def test_greedy_generation_through_the_entry_point(tmp_path, name):
         for index, token in enumerate(result.token_ids):
             row = logits[len(prompt) - 1 + index]
             assert row[token] >= row.max() - 1e-3 * row.abs().max(), f"token {index} is not the plain model's best"
+
+
+# ------------------------------------------------------------------ configurations drawn at random
+def drawn_configuration(seed):
+    """A configuration whose every size, option and order of layers is drawn: head sizes of 16 to 128 (also ones
+    no matrix-core kernel takes), one to six heads, values narrower and wider than keys, windows of 3 to 200 keys,
+    0 to 40 kept tokens, 0 to 5 taps, partial rotations with and without the ramp, latent ranks of 8 to 128 with
+    turned parts of 0 to 64, one to three state-space groups and norm parts, 2 to 9 experts, layers without a
+    feed-forward."""
+    import random
+    draw = random.Random(seed)
+    width = draw.choice([24, 40, 56, 64, 96])
+
+    def window():
+        return draw.choice([3, 8, 17, 33, 64, 100, 200])
+
+    def one_attention():
+        dim = draw.choice([16, 24, 48, 64, 80, 128])
+        G = draw.choice([1, 2, 3])
+        rot = draw.choice([0, dim, dim // 2 if (dim // 2) % 2 == 0 else dim])
+        scaling = draw.choice([None, (draw.choice([2.0, 4.0, 16.0]), draw.choice([16, 64, 256]), draw.choice([4.0, 16.0]), draw.choice([0.5, 1.0]))])
+        return pemarax_configs.attention(G * draw.choice([1, 2]), G, dim, draw.choice([dim, dim // 2, dim + 16]), window(),
+                                         draw.choice([0, 1, 7, 40]), draw.choice([0, 1, 2, 3, 5]), rot, scaling if rot else None,
+                                         base=draw.choice([100.0, 1e4, 1e6]), scale=draw.choice([None, 0.2]))
+
+    def one_latent():
+        rot_dim = draw.choice([0, 8, 32, 64])
+        return pemarax_configs.latent(draw.choice([1, 2, 5]), draw.choice([8, 16, 40]), rot_dim, draw.choice([8, 24, 48]),
+                                      draw.choice([8, 24, 64, 96, 128]), window(), draw.choice([None, rot_dim // 2]) if rot_dim >= 8 else None,
+                                      base=draw.choice([50.0, 1e5]))
+
+    def one_parallel():
+        G = draw.choice([1, 2])
+        dim = draw.choice([16, 48, 64, 128])
+        groups = draw.choice([1, 2, 3])
+        heads = groups * draw.choice([1, 2])
+        vdim = draw.choice([8, 16, 32, 64])
+        parts = draw.choice([1, 2, heads]) if (heads * vdim) % 2 == 0 else 1
+        return pemarax_configs.parallel((G * draw.choice([1, 3]), G, dim, draw.choice([dim, 2 * dim, 8]), window()),
+                                        (heads, vdim, draw.choice([8, 16, 32, 64]), groups, parts, draw.choice([2, 3, 4])))
+
+    layers = []
+    for _ in range(draw.choice([2, 3, 4])):
+        layer = draw.choice([one_attention, one_latent, one_parallel])()
+        experts = draw.choice([2, 3, 5, 9])
+        mlp = None if draw.random() < 0.25 else pemarax_configs.moe(experts, draw.randint(1, experts), draw.choice([8, 16, 40]))
+        layers.append(pemarax_configs.with_mlp(layer, mlp))
+    return {"architecture": "Pemarax", "width": width, "vocab": draw.choice([31, 100, 257]), "norm": {"eps": draw.choice([1e-5, 1e-6])},
+            "residual_mult": draw.choice([0.3, 0.5, 1.0, 1.4]), "layers": layers}
+
+
+DRAWN = [(seed, "float32") for seed in range(4100, 4116)] + [(seed, "bfloat16") for seed in (4102, 4104, 4106, 4110, 4113, 4115)]
+
+
+@pytest.mark.parametrize("seed, dtype", DRAWN)
+def test_randomly_drawn_configurations_whole_cut_and_side_by_side(tmp_path, seed, dtype):
+    """Whole, in portions beside another request's single tokens, and decoded: float32 at every position, bfloat16
+    (where head and state sizes that the matrix-core kernels take meet ones they do not) by the rounding gate."""
+    from macllm_infer_amd.engine import Engine, Lane
+    raw = drawn_configuration(seed)
+    raw, tensors = pemarax_configs.make_model_dir(raw, tmp_path, seed=seed,
+                                                  storage_dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    engine = Engine(str(tmp_path), dtype=dtype, device=DEV, kv_cache_block_tokens=draw_page(seed), kv_cache_capacity_tokens=640,
+                    max_active_sequences=3)
+    tokens, other = tokens_for(raw, 150, seed), tokens_for(raw, 30, seed + 1)
+    plain, beside = Plain(raw, tensors, tokens), Plain(raw, tensors, other)
+    engine.add_request("whole")
+    same(engine.step([Lane("whole", tokens, list(range(150)))]), plain, list(range(150)), dtype, f"seed {seed} whole")
+    engine.finish("whole")
+    engine.add_request("cut")
+    engine.add_request("other")
+    pieces, others, cursor, fed = [], [], 0, 0
+    for size in (5, 2, 40, 1, 1, 23, 64, 2, 12):
+        lanes = [Lane("cut", tokens[cursor:cursor + size], list(range(size)))]
+        if fed < 30:
+            count = 1 if fed else 4
+            lanes.append(Lane("other", other[fed:fed + count], list(range(count))))
+        got = engine.step(lanes)
+        pieces.append(got[:size])
+        if fed < 30:
+            others.append(got[size:])
+            fed += count
+        cursor += size
+    same(torch.cat(pieces), plain, list(range(150)), dtype, f"seed {seed} portions")
+    same(torch.cat(others), beside, list(range(fed)), dtype, f"seed {seed} the request beside")
+    engine.cache.check()
+
+
+def draw_page(seed):
+    return (4, 8, 16, 32)[seed % 4]
