@@ -118,7 +118,8 @@ class BlockTable:
 
     @property
     def first_live(self) -> int:
-        """Logical pages before this one were given back."""
+        """Logical pages before this one were given back (but for the pages of first tokens that the group's
+        window keeps)."""
         return native.lib().hc_first_live(self._core.pointer, self._group, self._slot)
 
     def live_pages(self) -> List[int]:

@@ -172,13 +172,20 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc,
       if (BIASED) {
         // the biased scores, already in units of log2 (the scale below is then one); a key past the column's
         // position gives a logarithm of anything, which the mask replaces
+        if (bias.on) {                 // the same for every lane
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float distance = (float)(col_pos[s] - (k0 + 16 * t + 4 * q + i));
-            score[t][i] = fmaf(score[t][i], scale_log2, -bias.r1[s] * __log2f(fmaf(bias.r2[s], fmaxf(distance, 0.f), 1.f)));
-          }
+            for (int i = 0; i < 4; ++i) {
+              const float distance = (float)(col_pos[s] - (k0 + 16 * t + 4 * q + i));
+              score[t][i] = fmaf(score[t][i], scale_log2, -bias.r1[s] * __log2f(fmaf(bias.r2[s], fmaxf(distance, 0.f), 1.f)));
+            }
+        } else {                       // a caller of this form for its sink alone: the scale, no logarithms
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) score[t][i] *= scale_log2;
+        }
       }
       if (MASKED) {
         // visible keys of the column: first_visible .. min(position, last_key); relative to the step

@@ -514,6 +514,47 @@ def test_windowed_attention_with_one_norm_weight_for_all_heads_alone(dtype, H, G
                    beside=rand(40, hidden, seed=3))
 
 
+@pytest.mark.parametrize("matrix", [False, True])
+@pytest.mark.parametrize("feed", ["whole", "decoded", "cut"])
+@pytest.mark.parametrize("distance, seen", [(1, True), (16, True), (52, True), (53, False), (54, False), (400, False)])
+def test_a_normed_key_counts_up_to_its_window_s_edge_and_not_beyond(distance, seen, feed, matrix):
+    """The left attention of a parallel layer, window 53, 500 tokens on pages of 16: the key projection is the query
+    projection of head 0 and both norms share a weight, so a row in the last row's direction has cosine one with the
+    last query whatever its length; four times as long, its value shows in the last row while the window holds it."""
+    hidden, T, window = 32, 500, 53
+    dim, vdim = (64, 128) if matrix else (16, 24)
+    spec, tensors, table, stored = normed_attention_parts(hidden, 2, 1, dim, vdim, window, 60)
+    table["scale"] = 12.0 / dim
+    from macllm_infer_amd.config.pemarax import _normed_attention
+    spec = _normed_attention(table, "left", 1e-5)
+    tensors["k_proj.weight"] = tensors["q_proj.weight"][:dim].clone()
+    stored["k"] = stored["q"][:dim].clone()
+    tensors["k_norm.weight"] = tensors["q_norm.weight"].clone()
+    stored["k.norm"] = stored["q.norm"].clone()
+    dtype = torch.bfloat16 if matrix else torch.float32
+    tensors, stored = rounded(tensors, dtype), rounded(stored, dtype)
+    names = {k: v.double() for k, v in stored.items()}
+    x = rand(T, hidden, seed=4).to(dtype).float()
+    target = T - 1 - distance
+    x[target] = 4.0 * x[T - 1]
+    want = pemarax_plain.windowed_attention(x.double(), table, names, 1e-5).float()
+    blind = x.clone()
+    blind[target] = -4.0 * x[T - 1]
+    without = pemarax_plain.windowed_attention(blind.double(), table, names, 1e-5).float()
+    share = float((want[-1] - without[-1]).abs().max() / want[-1].abs().max())
+    assert (share > 0.3) if seen else (share < 1e-6), f"the crafted key's share is {share}"
+    harness = PartHarness(spec, tensors, hidden, dtype, page_size=16, capacity=520)
+    if feed == "whole":
+        got = harness.run([("r", x)])[0][-1]
+    elif feed == "decoded":
+        harness.run([("r", x[:T - 1])])
+        got = harness.run([("r", x[T - 1:])])[0][-1]
+    else:
+        harness.run([("r", x[:target + 1])])
+        got = harness.run([("r", x[target + 1:])])[0][-1]
+    close(got, want[-1], dtype, f"distance {distance}")
+
+
 def state_space_parts(hidden, heads, vdim, state, groups, norm_groups, conv, seed):
     table = {"conv": conv, "groups": groups, "heads": heads, "norm_groups": norm_groups, "state": state, "vdim": vdim}
     from macllm_infer_amd.config.pemarax import _state_space
